@@ -16,7 +16,7 @@ from typing import Any, Optional
 @dataclass
 class ModelConfig:
     name: str
-    arch: str                       # "llama" | "gpt2" | "mixtral" | "nesizen" | "zinesun"
+    arch: str                       # "llama" | "gpt2" | "mixtral" | "nesizen" | "zinesun" | "lizizen"
     vocab_size: int
     hidden_size: int
     intermediate_size: int
@@ -42,6 +42,9 @@ class ModelConfig:
     residual_streams: int = 1       # > 1: hyper-connections (parallel residual streams)
     embed_scale: float = 1.0        # the embedding rows are multiplied by this
     conv_taps: int = 0              # > 1: causal per-channel convolution over time on a mixer's input
+    # layer indices in the order they run, when a span of layers repeats with the same weights
+    # (every run has its own cache and state); None: each layer once, in order
+    layer_runs: Optional[list] = None
 
     # ---- derived quantities ------------------------------------------------------------
     @property
@@ -95,7 +98,10 @@ class ModelConfig:
             return sum(sp["kv_heads"] * (sp["dim"] + sp["vdim"]) * dtype_bytes for sp in self.layer_specs
                        if sp["type"] == "attention" and sp["kv_from"] is None) + \
                 sum((2 * sp["kv_rank"] + sp["rot_dim"]) * dtype_bytes for sp in self.layer_specs
-                    if sp["type"] == "latent_attention")
+                    if sp["type"] == "latent_attention") + \
+                sum(sp["kv_heads"] * (sp["maps"] * sp["dim"] + sp["vdim"]) * dtype_bytes
+                    for sp in (self.layer_specs[i] for i in (self.layer_runs or range(len(self.layer_specs))))
+                    if sp["type"] in ("biased_attention", "diff_attention"))
         return 2 * self.num_layers * self.kv_size * dtype_bytes
 
     # ---- (de)serialisation -------------------------------------------------------------
@@ -163,6 +169,37 @@ class ModelConfig:
                    conv_taps=taps)
 
     @classmethod
+    def from_lizizen(cls, js: dict, name: str = "lizizen") -> "ModelConfig":
+        """Map a Lizizen config.json ("architecture": "Lizizen") to ModelConfig: parallel layers (mixer
+        and feed-forward read two norms of the same residual) with a token shift on the mixer's
+        input, softmax attention with a distance bias and a sink ("attention") or differential
+        attention over chunks ("attention_2"), clamped-GLU feed-forwards with biases, and a span of
+        layers that may run several times with the same weights ("loop"). Every size and per-layer
+        constant is taken from the file."""
+        kinds = {"attention": "biased_attention", "attention_2": "diff_attention"}
+        specs = []
+        for i, L in enumerate(js["layers"]):
+            if L["type"] not in kinds:
+                raise ValueError(f"layer {i}: Lizizen has no mixer {L['type']!r}")
+            specs.append(layer_spec(i, {**L, "type": kinds[L["type"]]}))
+        n = len(specs)
+        runs = list(range(n))
+        lp = js.get("loop")
+        if lp:
+            a, b, times = int(lp["start"]), int(lp["stop"]), int(lp.get("times", 1))
+            if not (0 <= a <= b <= n) or times < 1:
+                raise ValueError("loop: need 0 <= start <= stop <= layers and times >= 1")
+            runs = list(range(a)) + list(range(a, b)) * times + list(range(b, n))
+        mx = lambda key: max([sp.get(key) or 0 for sp in specs] + [0])  # noqa: E731
+        return cls(name=name, arch="lizizen", vocab_size=int(js["vocab"]), hidden_size=int(js["width"]),
+                   intermediate_size=max([sp["ffn"]["ff"] for sp in specs if sp["ffn"]] + [0]),
+                   num_layers=n, num_heads=max([sp["heads"] * sp["maps"] for sp in specs] + [0]),
+                   num_kv_heads=max(max([sp["kv_heads"] * sp["maps"] for sp in specs] + [0]), 1),
+                   head_dim=max(mx("dim"), mx("vdim")), max_position=1 << 30, norm_eps=float(js["norm"]["eps"]),
+                   norm="rms", act="glu_clamp", pos_emb="rope", tie_embeddings=False, bias=True,
+                   layer_specs=specs, layer_runs=runs)
+
+    @classmethod
     def from_model_dir(cls, path, name: Optional[str] = None) -> "ModelConfig":
         """config.json of a model folder -> ModelConfig; the "architecture" / "model_type" key
         chooses the family."""
@@ -173,6 +210,8 @@ class ModelConfig:
             return cls.from_nesizen(js, name=name)
         if family == "zinesun":
             return cls.from_zinesun(js, name=name)
+        if family == "lizizen":
+            return cls.from_lizizen(js, name=name)
         return cls.from_hf(js, name=name)
 
     @classmethod
@@ -215,12 +254,33 @@ def layer_spec(index: int, L: dict) -> dict:
     kv_from); "latent_attention": windowed softmax attention whose queries, keys and values are
     expanded from low-rank latents, with one rotated key part shared by the heads (heads, dim,
     rot_dim, vdim, kv_rank, q_rank, rot_base, scale, window); "gla": gated linear attention
-    (heads, dim, vdim, tau). `ffn`: None, or kind "dense" (ff) / "moe" (ff, limit or None for
-    unclamped experts, experts, top)."""
+    (heads, dim, vdim, tau); "biased_attention": causal softmax attention without rotation whose
+    scores lose a per-head logarithmic distance bias, with a zero-logit sink and a query
+    temperature that grows with the position (heads, kv_heads, dim, vdim, scale, qt_coef,
+    qt_every); "diff_attention": two softmax maps per head over the same values, combined as a
+    difference (heads, kv_heads, dim, vdim, maps = 2, scale, diff, chunk, rot_dims, rot_base,
+    softcap), with normed and half-rotated queries and keys, visible inside chunks of `chunk`
+    positions. `ffn`: None, or kind "dense" (ff) / "glu" (dense clamped GLU with biases: ff,
+    limit) / "moe" (ff, limit or None for unclamped experts, experts, top)."""
     m, t = L["mixer"], L["type"]
     sp = {"index": index, "type": t, "heads": int(m["heads"]), "dim": int(m["dim"]), "vdim": int(m["vdim"]),
-          "kv_from": None, "kv_heads": 0}
-    if t == "attention":
+          "kv_from": None, "kv_heads": 0, "maps": 1}
+    if t == "biased_attention":
+        qt = m.get("q_temp") or {"coef": 0.0, "every": 1}            # absent: no temperature
+        sp.update(kv_heads=int(m.get("kv_heads", m["heads"])), scale=float(m.get("scale", sp["dim"] ** -0.5)),
+                  qt_coef=float(qt.get("coef", 0.0)), qt_every=int(qt.get("every", 1)))
+        if sp["kv_heads"] < 1 or sp["heads"] % sp["kv_heads"] or sp["qt_every"] < 1:
+            raise ValueError(f"layer {index}: bad attention sizes")
+    elif t == "diff_attention":
+        rot = m.get("rot") or {"dims": 0, "base": 10000.0}          # absent: no rotation
+        mask = m.get("mask") or {"size": 1 << 30}                    # absent: plain causal attention
+        sp.update(kv_heads=int(m.get("kv_heads", m["heads"])), maps=2, scale=float(m.get("scale", sp["dim"] ** -0.5)),
+                  diff=float(m["diff"]), chunk=int(mask["size"]), rot_dims=int(rot["dims"]),
+                  rot_base=float(rot.get("base", 10000.0)), softcap=float(m.get("softcap") or 0.0))
+        if sp["kv_heads"] < 1 or sp["heads"] % sp["kv_heads"] or sp["rot_dims"] % 2 or sp["rot_dims"] > sp["dim"] \
+                or sp["chunk"] < 1 or sp["softcap"] < 0:
+            raise ValueError(f"layer {index}: bad differential-attention sizes")
+    elif t == "attention":
         rot = m.get("rot") or {"dims": 0, "base": 10000.0}          # absent: no rotation
         mask = m.get("mask") or {"size": 1 << 30}                    # absent: plain causal attention
         sp.update(kv_heads=int(m.get("kv_heads", m["heads"])), rot_dims=int(rot["dims"]),
@@ -249,6 +309,9 @@ def layer_spec(index: int, L: dict) -> dict:
     f = L.get("mlp")
     if f is None:
         sp["ffn"] = None
+    elif f["kind"] == "dense" and t in ("biased_attention", "diff_attention"):
+        lim = f.get("limit")
+        sp["ffn"] = {"kind": "glu", "ff": int(f["ff"]), "limit": float("inf") if lim is None else float(lim)}
     elif f["kind"] == "dense":
         sp["ffn"] = {"kind": "dense", "ff": int(f["ff"])}
     elif f["kind"] == "moe":
@@ -268,6 +331,10 @@ def layer_spec_params(h: int, sp: dict) -> int:
         n = h * H * D + H * Dv * h + H
         if sp["kv_from"] is None:
             n += h * sp["kv_heads"] * (D + Dv)
+    elif sp["type"] in ("biased_attention", "diff_attention"):
+        m = sp["maps"]
+        n = h * m * D * (H + sp["kv_heads"]) + h * sp["kv_heads"] * Dv + H * Dv * h + h
+        n += 2 * H if m == 1 else 6 * D + h * H * Dv
     elif sp["type"] == "latent_attention":
         R, Q, rd = sp["kv_rank"], sp["q_rank"], sp["rot_dim"]
         n = h * (Q + R + rd + H) + Q + R + Q * H * (D + rd) + R * H * (D + Dv) + H * Dv * h
@@ -275,7 +342,10 @@ def layer_spec_params(h: int, sp: dict) -> int:
         n = h * H * (2 * D + 2 * Dv) + H * Dv * h + Dv
     f = sp["ffn"]
     if f:
-        n += 2 * h * f["ff"] if f["kind"] == "dense" else f["experts"] * (3 * h * f["ff"] + h)
+        if f["kind"] == "glu":
+            n += 3 * h * f["ff"] + 2 * f["ff"] + h
+        else:
+            n += 2 * h * f["ff"] if f["kind"] == "dense" else f["experts"] * (3 * h * f["ff"] + h)
     return n + 2 * h
 
 

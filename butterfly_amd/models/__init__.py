@@ -1,10 +1,12 @@
 """Model families: Llama-3 (8B/70B), Mixtral 8x7B (MoE), GPT-2 — one shard-aware decoder — and
 Nesizen, a heterogeneous stack of attention / gated-linear-attention layers (models/nesizen.py),
-and Zinesun, latent-attention layers on a post-norm residual (models/zinesun.py)."""
+Zinesun, latent-attention layers on a post-norm residual (models/zinesun.py), and Lizizen, parallel
+layers with a token shift over distance-biased and differential attention (models/lizizen.py)."""
 from .shard import LocalDims, Shard, local_dims  # noqa: F401
 from .transformer import LogicalParam, TransformerLM  # noqa: F401
 from .nesizen import NesizenLM  # noqa: F401
 from .zinesun import ZinesunLM  # noqa: F401
+from .lizizen import LizizenLM  # noqa: F401
 
 
 class LlamaForCausalLM(TransformerLM):
@@ -20,7 +22,7 @@ class GPT2LMHeadModel(TransformerLM):
 
 
 _ARCH = {"llama": LlamaForCausalLM, "mixtral": MixtralForCausalLM, "gpt2": GPT2LMHeadModel,
-         "nesizen": NesizenLM, "zinesun": ZinesunLM}
+         "nesizen": NesizenLM, "zinesun": ZinesunLM, "lizizen": LizizenLM}
 
 
 def supports_f32(arch: str) -> bool:

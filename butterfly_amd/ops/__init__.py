@@ -837,18 +837,28 @@ def row_seq(row_cu, T: int):
 
 
 def attn_window_paged(q, k_cache, v_cache, tables, row_cu, positions, scale: float, window: int, keep_first: int,
-                      sink, row_map=None, out=None, fold_heads: bool = False, out_scale=None):
+                      sink, row_map=None, out=None, fold_heads: bool = False, out_scale=None, chunk: int = 0,
+                      softcap: float = 0.0, dist_bias=None, q_temp=None, maps: int = 1, out_dtype=None):
     """Windowed attention of packed rows over the paged cache with kept first positions and a
     sink logit (mixers.hip attn_window_paged_kernel; sink None: an ordinary softmax). `row_map`:
     ops.row_seq(row_cu, T), when the caller already has it. `out_scale` [T, H] f32 multiplies
     every head's output (an output gate). `fold_heads` (one shared key / value head only): the
     heads of a token become rows of the attention tiles, so a token's heads read each cached
-    page once instead of once per head."""
+    page once instead of once per head.
+
+    Score modifiers, applied in this order before the mask: `q_temp` (coef, every): the scale of a
+    row at position p is multiplied by 1 + coef ln(floor((p + 1) / every) + 1); `softcap` > 0:
+    s <- cap tanh(s / cap); `dist_bias` (a, b), f32 [H] each: s <- s - a[h] ln(1 + b[h] (p - j)).
+    `chunk` > 0 replaces the window: a row sees the keys of its own chunk of `chunk` positions
+    (counted from position 0). `maps` > 1: the key cache holds `maps` key heads per value head
+    (K [blocks, G * maps, BS, D]), the query heads are ordered (head, map), and query head (h, m)
+    reads key head (g(h), m) and value head g(h): several attention maps over the same values.
+    `out_dtype` torch.float32: the output keeps the f32 accumulator."""
     if not _gpu(q):
         return ref.attn_window_paged(q, k_cache, v_cache, tables, row_cu, positions, scale, window, keep_first, sink, out,
-                                     out_scale)
+                                     out_scale, chunk, softcap, dist_bias, q_temp, maps, out_dtype)
     if out is None:
-        out = _empty(q.shape[0], q.shape[1], v_cache.shape[2], dtype=q.dtype, device=q.device)
+        out = _empty(q.shape[0], q.shape[1], v_cache.shape[2], dtype=out_dtype or q.dtype, device=q.device)
     if row_map is None:
         row_map = row_seq(row_cu, q.shape[0])
     # steps of few rows (decoding): scratch so that several workgroups can share a tile's pages
@@ -856,8 +866,11 @@ def attn_window_paged(q, k_cache, v_cache, tables, row_cu, positions, scale: flo
     rows = q.shape[0] * q.shape[1]
     if q.dtype == torch.bfloat16 and rows <= 2048:
         part = _arena.get(q.device, "attn_window_part", 16 * rows * (v_cache.shape[2] + 2), torch.float32)
+    da, db = dist_bias if dist_bias is not None else (None, None)
+    qc, qe = q_temp if q_temp is not None else (0.0, 1)
     torch.ops.bfly.attn_window_paged(q, k_cache, v_cache, tables, row_map, row_cu, positions, float(scale), int(window),
-                                     int(keep_first), sink, out_scale, bool(fold_heads), part, out)
+                                     int(keep_first), sink, out_scale, bool(fold_heads), part, out, int(chunk),
+                                     float(softcap), da, db, float(qc), int(qe), int(maps))
     return out
 
 
@@ -1037,4 +1050,85 @@ def layer_norm_rows(x, w, b, eps: float, idx, out_dtype):
     R = x.shape[0] if idx is None else idx.numel()
     out = _empty(R, x.shape[1], dtype=out_dtype, device=x.device)
     torch.ops.bfly.layer_norm_rows(x, w, b, float(eps), idx, out)
+    return out
+
+
+# ---------------------------------------------------------------------------------------
+# Parallel layers with a token shift, differential attention, dense clamped GLU
+# (csrc/kernels/parlayer.hip)
+# ---------------------------------------------------------------------------------------
+def par_norm_shift(x, ya, yb, norm_a, norm_b, eps: float, offset: float, shift, state, state_slots, row_cu, positions,
+                   out_dtype, x_out=None, row_map=None):
+    """The step between two parallel layers, in one kernel: x' = x + (ya + yb) (the outputs of the
+    previous layer's mixer and feed-forward, either may be None; written to x_out, which must be
+    another buffer than x), then both inputs of the next layer from one RMS statistic of x':
+    ha = x' / rms (norm_a + offset) for the mixer and hb = x' / rms (norm_b + offset) for the
+    feed-forward (norm_b None: no hb). With `shift` [W] f32 the mixer's input is mixed with the
+    previous token's: ha + (prev - ha) shift, where prev is the unmixed ha of the row before in the
+    same sequence, state[slot] ([slots, W] f32) for a sequence's first row of the step, zero at
+    position 0; state[slot] then takes the unmixed ha of the sequence's last row. Returns
+    (x', ha, hb); x' is x itself when ya and yb are None."""
+    if not _gpu(x):
+        return ref.par_norm_shift(x, ya, yb, norm_a, norm_b, eps, offset, shift, state, state_slots, row_cu, positions,
+                                  out_dtype, x_out)
+    T, W = x.shape
+    if ya is None and yb is None:
+        x_out = None
+    elif x_out is None:
+        x_out = _empty(T, W, dtype=torch.float32, device=x.device)
+    ha = _empty(T, W, dtype=out_dtype, device=x.device)
+    hb = None if norm_b is None else _empty(T, W, dtype=out_dtype, device=x.device)
+    if row_map is None:
+        row_map = row_seq(row_cu, T)
+    torch.ops.bfly.par_norm_shift(x, ya, yb, x_out, norm_a, norm_b, float(eps), float(offset), shift,
+                                  state if shift is not None else None, state_slots if shift is not None else None,
+                                  row_map, row_cu, positions, ha, hb)
+    return (x if x_out is None else x_out), ha, hb
+
+
+def par_final(x, ya, yb, norm_w, eps: float, offset: float, idx, out_dtype):
+    """RMS norm with weight (w + offset) of rows idx (None: all) of x + (ya + yb): the last
+    parallel layer's residual sum fused with the output norm."""
+    if not _gpu(x):
+        return ref.par_final(x, ya, yb, norm_w, eps, offset, idx, out_dtype)
+    R = x.shape[0] if idx is None else idx.numel()
+    out = _empty(R, x.shape[1], dtype=out_dtype, device=x.device)
+    torch.ops.bfly.par_final(x, ya, yb, norm_w, float(eps), float(offset), idx, out)
+    return out
+
+
+def qk_norm_rope_kv(q, k, v, qn_w, kn_w, eps: float, positions, inv_freq, slots, k_cache, v_cache, q_out=None):
+    """Queries and keys prepared per head and the paged append, in one kernel: RMS norm over the
+    head with weight qn_w / kn_w [D] f32 (None: no norm), then rotation of the first 2 n dims
+    (n = len(inv_freq), may be 0) with dimension i paired with i + n by positions[t] * inv_freq[i].
+    q [T, Hq, D] -> q_out [T, Hq, Dp] (Dp = the key cache's row size, zero padded); k [T, Gk, D],
+    v [T, Gv, Dv] -> K [blocks, Gk, BS, Dp], V [blocks, Gv, Dvp, BS] at slots[t] >= 0 (the caches'
+    padding keeps the zeros it was allocated with). Returns q_out."""
+    if q_out is None:
+        q_out = _empty(q.shape[0], q.shape[1], k_cache.shape[3], dtype=q.dtype, device=q.device)
+    if not _gpu(q):
+        return ref.qk_norm_rope_kv(q, k, v, qn_w, kn_w, eps, positions, inv_freq, slots, k_cache, v_cache, q_out)
+    torch.ops.bfly.qk_norm_rope_kv(q, k, v, qn_w, kn_w, float(eps), positions, inv_freq, slots, k_cache, v_cache, q_out)
+    return q_out
+
+
+def diff_combine(a, lam: float, eps: float, out_mul: float, gate, Dv: int, out_dtype):
+    """Differential attention's combination: a [T, 2 H, >= Dv] f32 with heads ordered (head, map);
+    o = a[:, 2h] - lam a[:, 2h + 1] over the first Dv values, divided by its root mean square (eps
+    inside the root), times out_mul, times sigmoid(gate) (gate [T, H * Dv] logits; None: no
+    gate). Returns [T, H * Dv] in out_dtype."""
+    if not _gpu(a):
+        return ref.diff_combine(a, lam, eps, out_mul, gate, Dv, out_dtype)
+    out = _empty(a.shape[0], (a.shape[1] // 2) * Dv, dtype=out_dtype, device=a.device)
+    torch.ops.bfly.diff_combine(a, float(lam), float(eps), float(out_mul), gate, int(Dv), out)
+    return out
+
+
+def glu_clamp(gu, limit: float, alpha: float, up_offset: float):
+    """gu [T, 2 F] = [gate | up] (rows may be a view): g sigmoid(alpha g) (u + up_offset) with
+    g = min(gate, limit), u = clamp(up, -limit, limit) -> [T, F]."""
+    if not _gpu(gu):
+        return ref.glu_clamp(gu, limit, alpha, up_offset)
+    out = _empty(gu.shape[0], gu.shape[1] // 2, dtype=gu.dtype, device=gu.device)
+    torch.ops.bfly.glu_clamp(gu, float(limit), float(alpha), float(up_offset), out)
     return out

@@ -610,13 +610,21 @@ def rope_partial_kv(q, k, v, positions, inv_freq, slots, k_cache, v_cache):
 
 
 def attn_window_paged(q, k_cache, v_cache, tables, row_cu, positions, scale, window, keep_first, sink, out=None,
-                      out_scale=None):
+                      out_scale=None, chunk=0, softcap=0.0, dist_bias=None, q_temp=None, maps=1, out_dtype=None):
     """Row r of sequence s (rows row_cu[s] .. row_cu[s+1]) at position p attends to the cached
     keys j <= p of tables[s] with p - j < window or j < keep_first; the softmax denominator
     also holds exp(sink[h]) (sink None: an ordinary softmax). out_scale [T, H] f32: every head's
-    output is multiplied by its entry (an output gate)."""
+    output is multiplied by its entry (an output gate). chunk > 0: instead of the window, the
+    keys of the row's own chunk of `chunk` positions (j >= p - p % chunk). q_temp (coef, every):
+    the score is multiplied by 1 + coef ln(floor((p + 1) / every) + 1); softcap > 0: s <- cap
+    tanh(s / cap); dist_bias (a, b) [H] f32: s <- s - a[h] ln(1 + b[h] (p - j)), in that order.
+    maps > 1: the key cache holds `maps` key heads per value head, and query head h reads key
+    head ((h / maps) / R) * maps + h % maps (R query-head groups per value head) and its value
+    head."""
     T, H, D = q.shape
-    G, bs, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[2]
+    Gk, bs, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[2]
+    G = v_cache.shape[1]
+    R = (H // maps) // G
     o = torch.zeros(T, H, Dv, dtype=torch.float32, device=q.device)
     cu = row_cu.tolist()
     pos = positions.tolist()
@@ -626,15 +634,25 @@ def attn_window_paged(q, k_cache, v_cache, tables, row_cu, positions, scale, win
         pmax = max(pos[cu[s]:cu[s + 1]])
         nb = pmax // bs + 1
         blk = tables[s, :nb].long()
-        K = k_cache[blk].float().permute(1, 0, 2, 3).reshape(G, nb * bs, D)
+        K = k_cache[blk].float().permute(1, 0, 2, 3).reshape(Gk, nb * bs, D)
         V = v_cache[blk].float().permute(1, 0, 3, 2).reshape(G, nb * bs, Dv)
         j = torch.arange(nb * bs, device=q.device)[None, :]
         p = positions[cu[s]:cu[s + 1]].long()[:, None]
         ok = (j <= p) & ((p - j < window) | (j < keep_first))
+        if chunk > 0:
+            ok = (j <= p) & ((j >= p - p % chunk) | (j < keep_first))
         qs = q[cu[s]:cu[s + 1]].float()
+        rs = torch.full_like(p, scale, dtype=torch.float32)
+        if q_temp is not None:
+            rs = rs * (1.0 + q_temp[0] * torch.log(torch.floor((p + 1).float() / q_temp[1]) + 1.0))
         for h in range(H):
-            g = h // (H // G)
-            sc = (qs[:, h] @ K[g].t()) * scale
+            gk = ((h // maps) // R) * maps + h % maps
+            g = gk // maps
+            sc = (qs[:, h] @ K[gk].t()) * rs
+            if softcap > 0:
+                sc = softcap * torch.tanh(sc / softcap)
+            if dist_bias is not None:
+                sc = sc - dist_bias[0][h].float() * torch.log1p(dist_bias[1][h].float() * (p - j).clamp(min=0).float())
             sc = sc.masked_fill(~ok, float("-inf"))
             if sink is None:
                 w = torch.softmax(sc, -1)
@@ -644,7 +662,7 @@ def attn_window_paged(q, k_cache, v_cache, tables, row_cu, positions, scale, win
             o[cu[s]:cu[s + 1], h] = w @ V[g]
     if out_scale is not None:
         o = o * out_scale.float()[:, :, None]
-    o = o.to(q.dtype)
+    o = o.to(out_dtype or q.dtype)
     if out is None:
         return o
     out.copy_(o)
@@ -854,3 +872,102 @@ def layer_norm_rows(x, w, b, eps, idx, out_dtype):
     """Layer norm (weight and bias, f32) of rows idx of x (None: all rows)."""
     xs = x if idx is None else x[idx.long()]
     return _layer_norm_f32(xs, w, b, eps).to(out_dtype)
+
+
+# ---------------------------------------------------------------------------------------
+# Parallel layers with a token shift; differential attention; dense clamped GLU
+# ---------------------------------------------------------------------------------------
+def par_norm_shift(x, ya, yb, norm_a, norm_b, eps, offset, shift, state, state_slots, row_cu, positions, out_dtype,
+                   x_out=None):
+    """x' = x + (ya + yb) (f32; either may be None), n = x' / rms(x'), ha = n (norm_a + offset) mixed
+    with the previous token's unmixed ha (ha + (prev - ha) shift; zeros before position 0; for a
+    sequence's first row of the step: state[slot]), hb = n (norm_b + offset). state[slot] <- the
+    unmixed ha of the sequence's last row. Returns (x', ha, hb); hb None without norm_b."""
+    xn = x.float()
+    if ya is not None or yb is not None:
+        y = (ya.float() if ya is not None else 0) + (yb.float() if yb is not None else 0)
+        xn = xn + y
+    if x_out is not None and xn is not x:
+        x_out.copy_(xn)
+        xn = x_out
+    n = xn * torch.rsqrt(xn.pow(2).mean(-1, keepdim=True) + eps)
+    ha = n * (norm_a.float() + offset)
+    hb = None if norm_b is None else (n * (norm_b.float() + offset)).to(out_dtype)
+    if shift is not None:
+        prev = torch.zeros_like(ha)
+        prev[1:] = ha[:-1]
+        cu, pos = row_cu.tolist(), positions.tolist()
+        sl = state_slots.tolist()
+        for s in range(len(cu) - 1):
+            a, b = cu[s], cu[s + 1]
+            if b <= a:
+                continue
+            if pos[a] > 0 and sl[s] >= 0:
+                prev[a] = state[sl[s]]
+            else:
+                prev[a] = 0
+            if sl[s] >= 0:
+                state[sl[s]] = ha[b - 1]
+        ha = ha + (prev - ha) * shift.float()
+    return xn, ha.to(out_dtype), hb
+
+
+def par_final(x, ya, yb, norm_w, eps, offset, idx, out_dtype):
+    """RMS norm with weight (w + offset) of rows idx (None: all) of x + (ya + yb)."""
+    sel = (lambda t: t) if idx is None else (lambda t: t[idx.long()])
+    xn = sel(x).float()
+    if ya is not None or yb is not None:
+        xn = xn + ((sel(ya).float() if ya is not None else 0) + (sel(yb).float() if yb is not None else 0))
+    return _rms_offset(xn, norm_w, eps, offset).to(out_dtype)
+
+
+def qk_norm_rope_kv(q, k, v, qn_w, kn_w, eps, positions, inv_freq, slots, k_cache, v_cache, q_out):
+    """Per head: RMS norm over the head with weight qn_w / kn_w [D] (None: no norm), then rotation
+    of the first 2 n dims (n = len(inv_freq)) with dimension i paired with i + n, angle position *
+    inv_freq[i] (f32). q [T, Hq, D] -> q_out [T, Hq, >= D] (zero padded); k [T, Gk, D], v [T, Gv,
+    Dv] -> cache rows K [blocks, Gk, BS, >= D], V [blocks, Gv, >= Dv, BS] at slots[t] >= 0."""
+    n = inv_freq.numel()
+    a = positions.float()[:, None] * inv_freq.float()[None]
+    c, s = torch.cos(a)[:, None, :], torch.sin(a)[:, None, :]
+
+    def prep(t, w):
+        tf = t.float()
+        if w is not None:
+            tf = tf * torch.rsqrt(tf.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+        if n:
+            u, z = tf[..., :n], tf[..., n:2 * n]
+            tf = torch.cat([u * c - z * s, z * c + u * s, tf[..., 2 * n:]], -1)
+        return tf
+
+    D, Dv = q.shape[2], v.shape[2]
+    q_out.zero_()
+    q_out[..., :D] = prep(q, qn_w).to(q_out.dtype)
+    kk = prep(k, kn_w)
+    bs = k_cache.shape[2]
+    ok = slots >= 0
+    sl = slots[ok].long()
+    k_cache[sl // bs, :, sl % bs, :D] = kk[ok].to(k_cache.dtype)
+    v_cache[sl // bs, :, :Dv, sl % bs] = v[ok].to(v_cache.dtype)
+    return q_out
+
+
+def diff_combine(a, lam, eps, out_mul, gate, Dv, out_dtype):
+    """a [T, 2 H, >= Dv] f32, heads ordered (head, map): o = a[:, 2h] - lam a[:, 2h + 1] over the
+    first Dv values, divided by its root mean square (eps inside the root), times out_mul, times
+    sigmoid(gate) (gate [T, H * Dv] logits, None: no gate). Returns [T, H * Dv]."""
+    T, H2 = a.shape[0], a.shape[1]
+    af = a.float()[..., :Dv]
+    o = af[:, 0::2] - lam * af[:, 1::2]
+    o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * out_mul
+    o = o.reshape(T, (H2 // 2) * Dv)
+    if gate is not None:
+        o = o * torch.sigmoid(gate.float())
+    return o.to(out_dtype)
+
+
+def glu_clamp(gu, limit, alpha, up_offset, out_dtype=None):
+    """gu [T, 2 F] = [gate | up]: min(g, limit) sigmoid(alpha min(g, limit)) (clamp(u, +-limit) + up_offset)."""
+    F = gu.shape[1] // 2
+    g = gu[:, :F].float().clamp(max=limit)
+    u = gu[:, F:].float().clamp(min=-limit, max=limit)
+    return (g * torch.sigmoid(alpha * g) * (u + up_offset)).to(out_dtype or gu.dtype)

@@ -172,18 +172,37 @@ void row_seq(const Tensor& row_cu, Tensor& out) {
 void attn_window_paged(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache, const Tensor& tables,
                        const Tensor& row_seq_t, const Tensor& row_cu, const Tensor& positions, double scale,
                        int64_t window, int64_t keep_first, const optional<Tensor>& sink,
-                       const optional<Tensor>& out_scale, bool fold_heads, const optional<Tensor>& part, Tensor& out) {
-  CHK_GPU(q); CHK_HEADS(q); CHK_SAME(k_cache, q); CHK_SAME(v_cache, q); CHK_SAME(out, q);
+                       const optional<Tensor>& out_scale, bool fold_heads, const optional<Tensor>& part, Tensor& out,
+                       int64_t chunk, double softcap, const optional<Tensor>& dist_a, const optional<Tensor>& dist_b,
+                       double qt_coef, int64_t qt_every, int64_t maps) {
+  CHK_GPU(q); CHK_HEADS(q); CHK_SAME(k_cache, q); CHK_SAME(v_cache, q);
+  bfly::AttnMod md;
+  md.out_f32 = out.scalar_type() == at::kFloat && !is_f32(q);
+  TORCH_CHECK(md.out_f32 || out.scalar_type() == q.scalar_type(), "attn_window_paged: out must be f32 or of q's type");
+  TORCH_CHECK(chunk >= 0 && softcap >= 0 && qt_every >= 1 && maps >= 1, "attn_window_paged: modifiers");
+  md.chunk = (int)chunk;
+  md.softcap = (float)softcap;
+  md.qt_coef = (float)qt_coef;
+  md.qt_every = (int)qt_every;
+  md.maps = (int)maps;
   CHK_I32(tables); CHK_I32(row_seq_t); CHK_I32(positions);
   const int64_t T = q.size(0), H = q.size(1), D = q.size(2);
   TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.is_contiguous() && v_cache.is_contiguous(),
               "attn_window_paged: caches");
-  const int64_t G = k_cache.size(1), bs = k_cache.size(2), Dv = v_cache.size(2);
-  TORCH_CHECK(k_cache.size(3) == D && v_cache.size(1) == G && v_cache.size(3) == bs && v_cache.size(0) == k_cache.size(0),
-              "attn_window_paged: cache shapes K [blocks, G, BS, D], V [blocks, G, Dv, BS]");
+  const int64_t G = v_cache.size(1), bs = k_cache.size(2), Dv = v_cache.size(2);
+  TORCH_CHECK(k_cache.size(3) == D && k_cache.size(1) == G * maps && v_cache.size(3) == bs &&
+                  v_cache.size(0) == k_cache.size(0),
+              "attn_window_paged: cache shapes K [blocks, G * maps, BS, D], V [blocks, G, Dv, BS]");
   CHK_I32(row_cu);
   TORCH_CHECK(row_cu.numel() == tables.size(0) + 1, "attn_window_paged: row_cu");
-  TORCH_CHECK(G > 0 && H % G == 0 && Dv <= 512 && D <= 4096, "attn_window_paged: head counts / sizes");
+  TORCH_CHECK(G > 0 && H % (G * maps) == 0 && Dv <= 512 && D <= 4096, "attn_window_paged: head counts / sizes");
+  TORCH_CHECK(dist_a.has_value() == dist_b.has_value(), "attn_window_paged: the distance bias needs both vectors");
+  if (dist_a.has_value()) {
+    CHK_F32(*dist_a); CHK_F32(*dist_b);
+    TORCH_CHECK(dist_a->numel() == H && dist_b->numel() == H, "attn_window_paged: distance bias [H]");
+    md.dist_a = dist_a->data_ptr<float>();
+    md.dist_b = dist_b->data_ptr<float>();
+  }
   TORCH_CHECK(tables.dim() == 2 && row_seq_t.numel() == T && positions.numel() == T, "attn_window_paged: index shapes");
   const float *sinkp = nullptr, *gatep = nullptr;
   if (sink.has_value()) {
@@ -212,13 +231,13 @@ void attn_window_paged(const Tensor& q, const Tensor& k_cache, const Tensor& v_c
                                                   (int)tables.size(0), positions.data_ptr<int>(), (float)scale,
                                                   (int)window, (int)keep_first, sinkp, gatep, out.data_ptr(),
                                                   (int)T, (int)H, (int)G, (int)D, (int)Dv, (int)bs, fold_heads, partp,
-                                                  (long)part_n, cur_stream()))
+                                                  (long)part_n, cur_stream(), md))
     return;
   bfly::launch_attn_window_paged(q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
                                  tables.data_ptr<int>(), (int)tables.size(1), row_seq_t.data_ptr<int>(),
                                  (int)tables.size(0), positions.data_ptr<int>(), (float)scale, (int)window,
                                  (int)keep_first, sinkp, gatep, out.data_ptr(), (int)T, (int)H, (int)G, (int)D,
-                                 (int)Dv, (int)bs, is_f32(q), cur_stream());
+                                 (int)Dv, (int)bs, is_f32(q), cur_stream(), md);
 }
 
 void gla_scan(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor& z, Tensor& state,
@@ -342,7 +361,8 @@ TORCH_LIBRARY_FRAGMENT(bfly, m) {
   m.def("row_seq(Tensor row_cu, Tensor(a!) out) -> ()");
   m.def("attn_window_paged(Tensor q, Tensor k_cache, Tensor v_cache, Tensor tables, Tensor row_seq, Tensor row_cu, "
         "Tensor positions, float scale, int window, int keep_first, Tensor? sink, Tensor? out_scale, bool fold_heads, "
-        "Tensor(b!)? part, Tensor(a!) out) -> ()");
+        "Tensor(b!)? part, Tensor(a!) out, int chunk=0, float softcap=0., Tensor? dist_a=None, Tensor? dist_b=None, "
+        "float qt_coef=0., int qt_every=1, int maps=1) -> ()");
   m.def("gla_scan(Tensor q, Tensor k, Tensor v, Tensor z, Tensor(a!) state, Tensor state_slots, Tensor row_cu, "
         "Tensor positions, float tau, float q_scale, Tensor(b!) o) -> ()");
   m.def("gla_out(Tensor o, Tensor g, Tensor norm_w, float eps, Tensor(a!) out) -> ()");

@@ -47,6 +47,21 @@ void launch_rope_partial_kv(void* q, long q_ld, void* k, long k_ld, const void* 
                             int T, int H, int G, int D, int Dv, int block_size, bool f32, hipStream_t s);
 // row_seq[t] = the sequence whose row range [row_cu[s], row_cu[s+1]) holds row t, else -1
 void launch_row_seq(const int* row_cu, int nseq, int* row_seq, int T, hipStream_t s);
+// Score modifiers of the paged attention kernels, all off by default. Order: scale (with the
+// temperature), cap, distance bias, mask.
+struct AttnMod {
+  int chunk = 0;                  // > 0: instead of the window, a row sees its own chunk of `chunk` positions
+                                  // (j >= p - p % chunk)
+  float softcap = 0.f;            // > 0: s <- cap tanh(s / cap)
+  const float* dist_a = nullptr;  // [H] (with dist_b): s <- s - a[h] ln(1 + b[h] (p - j))
+  const float* dist_b = nullptr;
+  float qt_coef = 0.f;            // the score scale of a row at p is multiplied by
+  int qt_every = 1;               // 1 + coef ln(floor((p + 1) / every) + 1)
+  int maps = 1;                   // key heads per value head: K [blocks, G * maps, BS, D]; query heads are ordered
+                                  // (head, map) and head (h, m) reads key head (g(h), m) and value head g(h)
+  bool out_f32 = false;           // out is float whatever the inputs
+};
+
 // Row t of sequence row_seq[t] (-1: padding row, output zero) at position p sees cached keys
 // j <= p with p - j < window or j < keep_first; the softmax denominator includes exp(sink[h])
 // (sink == nullptr: an ordinary softmax); out_scale (nullable) [T, H] multiplies each head's output.
@@ -54,7 +69,8 @@ void launch_row_seq(const int* row_cu, int nseq, int* row_seq, int T, hipStream_
 void launch_attn_window_paged(const void* q, long q_ld, const void* k_cache, const void* v_cache, const int* tables,
                               int max_blocks, const int* row_seq, int nseq, const int* positions, float scale,
                               int window, int keep_first, const float* sink, const float* out_scale, void* out, int T,
-                              int H, int G, int D, int Dv, int block_size, bool f32, hipStream_t s);
+                              int H, int G, int D, int Dv, int block_size, bool f32, hipStream_t s,
+                              const AttnMod& md = AttnMod());
 
 // The MFMA form of launch_attn_window_paged over row_cu (bf16, 32-token pages, D and Dv in {32, 64,
 // 96, 128, 192, 256}, 16-byte aligned q rows): false if the shape has no such form. `fold` (G == 1):
@@ -64,7 +80,8 @@ void launch_attn_window_paged(const void* q, long q_ld, const void* k_cache, con
 bool launch_attn_window_mfma(const void* q, long q_ld, const void* k_cache, const void* v_cache, const int* tables,
                              int max_blocks, const int* row_cu, int nseq, const int* positions, float scale, int window,
                              int keep_first, const float* sink, const float* out_scale, void* out, int T, int H, int G,
-                             int D, int Dv, int block_size, bool fold, float* part, long part_floats, hipStream_t s);
+                             int D, int Dv, int block_size, bool fold, float* part, long part_floats, hipStream_t s,
+                             const AttnMod& md = AttnMod());
 
 // Gated linear attention scan over packed rows (see ops.gla_scan). Returns < 0 if D > 256.
 int launch_gla_scan(const void* q, long q_ld, const void* k, long k_ld, const void* v, long v_ld, const void* z,

@@ -67,6 +67,22 @@ __global__ __launch_bounds__(256) void rope_partial_kv_kernel(T* __restrict__ q,
 // of every (row, head): an output gate.
 constexpr int kMaxDvLane = 8;
 
+// Score modifiers shared by the attention kernels (AttnMod): the lowest visible position of a row
+// outside the kept prefix, the row's score scale, and the capped / distance-biased score.
+__device__ __forceinline__ int attn_row_lo(int p, int window, int chunk) {
+  return chunk > 0 ? p - p % chunk : max(0, p - window + 1);
+}
+__device__ __forceinline__ float attn_row_scale(int p, float scale, const AttnMod& md) {
+  if (md.qt_coef == 0.f) return scale;
+  return scale * (1.f + md.qt_coef * logf((float)((p + 1) / md.qt_every) + 1.f));
+}
+__device__ __forceinline__ float attn_score(float dot, float rscale, int dist, float da, float db, const AttnMod& md) {
+  float sc = dot * rscale;
+  if (md.softcap > 0.f) sc = md.softcap * tanhf(sc / md.softcap);
+  if (md.dist_a) sc -= da * log1pf(db * (float)dist);
+  return sc;
+}
+
 template <typename T>
 __global__ __launch_bounds__(64) void attn_window_paged_kernel(const T* __restrict__ q, long q_ld,
                                                                const T* __restrict__ k_cache,
@@ -77,25 +93,35 @@ __global__ __launch_bounds__(64) void attn_window_paged_kernel(const T* __restri
                                                                int window, int keep_first,
                                                                const float* __restrict__ sink,
                                                                const float* __restrict__ out_scale,
-                                                               T* __restrict__ out, int H, int G, int D, int Dv,
-                                                               int bs) {
+                                                               void* __restrict__ out_v, int H, int G, int D, int Dv,
+                                                               int bs, AttnMod md) {
   extern __shared__ float smem[];      // q [D] | p [64] | key row base index [64] (as int)
   float* sq = smem;
   float* sp = smem + D;
   long* sj = reinterpret_cast<long*>(smem + D + 64 + ((D & 1) ? 1 : 0));
   const long t = blockIdx.x;
   const int h = blockIdx.y, lane = threadIdx.x;
-  const int g = h / (H / G);
+  // G value heads; md.maps key heads per value head, query heads ordered (head, map)
+  const int Gk = G * md.maps;
+  const int gk = ((h / md.maps) / ((H / md.maps) / G)) * md.maps + h % md.maps;
+  const int g = gk / md.maps;
   const int s = row_seq[t];
+  T* out = reinterpret_cast<T*>(out_v);
+  float* outf = reinterpret_cast<float*>(out_v);
   if (s < 0) {       // padding row of a fixed-shape step
-    for (int d = lane; d < Dv; d += 64) out[(t * H + h) * Dv + d] = (T)0.f;
+    for (int d = lane; d < Dv; d += 64) {
+      if (md.out_f32) outf[(t * H + h) * Dv + d] = 0.f;
+      else out[(t * H + h) * Dv + d] = (T)0.f;
+    }
     return;
   }
   const int p = positions[t];
+  const float rscale = attn_row_scale(p, scale, md);
+  const float da = md.dist_a ? md.dist_a[h] : 0.f, db = md.dist_a ? md.dist_b[h] : 0.f;
   const int* tab = tables + (long)s * max_blocks;
   for (int d = lane; d < D; d += 64) sq[d] = (float)q[t * q_ld + (long)h * D + d];
   __syncthreads();
-  const int lo = max(0, p - window + 1);
+  const int lo = attn_row_lo(p, window, md.chunk);
   const int n1 = min(keep_first, lo);          // kept first positions outside the window
   const int total = n1 + (p - lo + 1);
   float m = sink ? sink[h] : -1e30f, l = sink ? 1.f : 0.f;
@@ -106,12 +132,12 @@ __global__ __launch_bounds__(64) void attn_window_paged_kernel(const T* __restri
     long kv_row = 0;      // index of V^T[0][key] of this lane's key
     if (i < total) {
       const int j = i < n1 ? i : lo + (i - n1);
-      const long pg = (long)tab[j / bs] * G + g;
-      kv_row = pg * Dv * bs + (j % bs);
-      const T* kr = k_cache + (pg * bs + (j % bs)) * D;
+      const long blk = tab[j / bs];
+      kv_row = (blk * G + g) * Dv * bs + (j % bs);
+      const T* kr = k_cache + ((blk * Gk + gk) * bs + (j % bs)) * D;
       float a = 0.f;
       for (int d = 0; d < D; ++d) a = fmaf(sq[d], (float)kr[d], a);
-      sc = a * scale;
+      sc = attn_score(a, rscale, p - j, da, db, md);
     }
     const float mn = fmaxf(m, wave_max(sc));
     const float pe = i < total ? expf(sc - mn) : 0.f;
@@ -136,7 +162,10 @@ __global__ __launch_bounds__(64) void attn_window_paged_kernel(const T* __restri
 #pragma unroll
   for (int c = 0; c < kMaxDvLane; ++c) {
     const int d = lane + 64 * c;
-    if (d < Dv) out[(t * H + h) * Dv + d] = (T)(acc[c] * inv);
+    if (d < Dv) {
+      if (md.out_f32) outf[(t * H + h) * Dv + d] = acc[c] * inv;
+      else out[(t * H + h) * Dv + d] = (T)(acc[c] * inv);
+    }
   }
 }
 
@@ -166,9 +195,9 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __res
                                                                int window, int keep_first,
                                                                const float* __restrict__ sink,
                                                                const float* __restrict__ out_scale,
-                                                               bf16* __restrict__ out, int H, int G, int fold,
+                                                               void* __restrict__ out_v, int H, int G, int fold,
                                                                int nsplit, float* __restrict__ part,
-                                                               long part_rows) {
+                                                               long part_rows, AttnMod md) {
   constexpr int D = 32 * DS, Dv = 16 * DVT, BS = 32;
   const int split = blockIdx.z;
   extern __shared__ float smem[];          // o of waves 1-3 [3][DVT][4][64] | m [3][16] | l [3][16]
@@ -191,8 +220,14 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __res
   const long frow = rv ? row0 + qr : row0;
   const long row = frow / rf;                                   // the token's row
   const int h = fold > 0 ? (int)(frow % rf) : (int)blockIdx.y;  // this lane's query head
-  const int g = fold > 0 ? 0 : h / (H / G);
+  // G value heads; md.maps key heads per value head, query heads ordered (head, map)
+  const int Gk = G * md.maps;
+  const int gk = fold > 0 ? 0 : ((h / md.maps) / ((H / md.maps) / G)) * md.maps + h % md.maps;
+  const int g = gk / md.maps;
   const int p = rv ? positions[row] : -1;
+  const int plo = attn_row_lo(max(p, 0), window, md.chunk);
+  const float rscale = attn_row_scale(max(p, 0), scale, md);
+  const float da = md.dist_a ? md.dist_a[h] : 0.f, db = md.dist_a ? md.dist_b[h] : 0.f;
   int pmin = rv ? p : 0x7fffffff, pmax = p;
 #pragma unroll
   for (int o = 1; o < 16; o <<= 1) {
@@ -210,13 +245,13 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __res
 #pragma unroll
   for (int t = 0; t < DVT; ++t) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int kp = (min(keep_first, pmax + 1) + BS - 1) / BS;          // pages of the kept prefix
-  const int wp0 = max(max(0, pmin - window + 1) / BS, kp), wp1 = pmax / BS;
+  const int wp0 = max(attn_row_lo(pmin, window, md.chunk) / BS, kp), wp1 = pmax / BS;
   const int npages = kp + max(0, wp1 - wp0 + 1);
   auto page_of = [&](int i) { return i < kp ? i : wp0 + (i - kp); };
   auto load_kv = [&](int pg, bf16x8 (&kf)[2][DS], bf16x8 (&vf)[DVT]) {
-    const long blk = (long)tab[pg] * G + g;
-    const bf16* Kp = k_cache + blk * BS * D;
-    const bf16* Vp = v_cache + blk * Dv * BS;
+    const long blk = tab[pg];
+    const bf16* Kp = k_cache + (blk * Gk + gk) * BS * D;
+    const bf16* Vp = v_cache + (blk * G + g) * Dv * BS;
 #pragma unroll
     for (int kh = 0; kh < 2; ++kh)
 #pragma unroll
@@ -252,8 +287,8 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __res
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int j = pg * BS + 16 * kh + 4 * gg + i;
-        const bool ok = j <= p && (p - j < window || j < keep_first);
-        sc[4 * kh + i] = ok ? st[kh][i] * scale : -INFINITY;
+        const bool ok = j <= p && (j >= plo || j < keep_first);
+        sc[4 * kh + i] = ok ? attn_score(st[kh][i], rscale, p - j, da, db, md) : -INFINITY;
         mx = fmaxf(mx, sc[4 * kh + i]);
       }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
@@ -325,7 +360,15 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __res
     return;
   }
   const float inv = (out_scale ? out_scale[row * H + h] : 1.f) / l;
-  bf16* orow = out + (row * H + h) * Dv;
+  if (md.out_f32) {
+    float* orow = reinterpret_cast<float*>(out_v) + (row * H + h) * Dv;
+#pragma unroll
+    for (int t = 0; t < DVT; ++t)
+      *reinterpret_cast<f32x4*>(orow + 16 * t + 4 * gg) =
+          f32x4{o[t][0] * inv, o[t][1] * inv, o[t][2] * inv, o[t][3] * inv};
+    return;
+  }
+  bf16* orow = reinterpret_cast<bf16*>(out_v) + (row * H + h) * Dv;
 #pragma unroll
   for (int t = 0; t < DVT; ++t) {
     bf16x4 w;
@@ -491,7 +534,7 @@ __global__ __launch_bounds__(256) void attn_fold_tile_kernel(const bf16* __restr
 // One wave per (row, head): fold the nsplit partial results part[split][row][o (Dv) | m | l].
 __global__ __launch_bounds__(64) void attn_split_merge_kernel(const float* __restrict__ part, long part_rows,
                                                               int nsplit, const float* __restrict__ out_scale,
-                                                              bf16* __restrict__ out, int Dv) {
+                                                              void* __restrict__ out_v, int Dv, bool out_f32) {
   const long r = blockIdx.x;
   const int lane = threadIdx.x;
   float m = -1e30f;
@@ -508,7 +551,8 @@ __global__ __launch_bounds__(64) void attn_split_merge_kernel(const float* __res
       const float* pp = part + ((long)s * part_rows + r) * (Dv + 2);
       a += pp[d] * __expf(pp[Dv] - m);
     }
-    out[r * Dv + d] = (bf16)(a * inv);
+    if (out_f32) reinterpret_cast<float*>(out_v)[r * Dv + d] = a * inv;
+    else reinterpret_cast<bf16*>(out_v)[r * Dv + d] = (bf16)(a * inv);
   }
 }
 
@@ -669,8 +713,8 @@ void launch_row_seq(const int* row_cu, int nseq, int* row_seq, int T, hipStream_
 template <int DS>
 static bool attn_mfma_dv(const bf16* q, long q_ld, const bf16* kc, const bf16* vc, const int* tables, int max_blocks,
                          const int* row_cu, int nseq, const int* positions, float scale, int window, int keep_first,
-                         const float* sink, const float* out_scale, bf16* out, int T, int H, int G, int Dv, bool fold,
-                         int nsplit, float* part, hipStream_t s) {
+                         const float* sink, const float* out_scale, void* out, int T, int H, int G, int Dv, bool fold,
+                         int nsplit, float* part, hipStream_t s, const AttnMod& md) {
   if (fold && (long)T * H >= 2048 && (long)T * H >= 128L * nseq) {
     // many rows per sequence (prompts): 64-row tiles over pages staged in LDS
     const unsigned tiles = (unsigned)(((long)T * H + 63) / 64 + nseq);
@@ -685,7 +729,7 @@ static bool attn_mfma_dv(const bf16* q, long q_ld, const bf16* kc, const bf16* v
     }                                                                                                         \
     attn_fold_tile_kernel<DS, DVT><<<tiles, 256, lds, s>>>(q, q_ld, kc, vc, tables, max_blocks, row_cu, nseq,   \
                                                           positions, scale, window, keep_first, sink, out_scale, \
-                                                          out, H);                                            \
+                                                          (bf16*)out, H);                                            \
   }
     switch (Dv) {
       case 32: BFLY_ATF(2); return true;
@@ -705,7 +749,7 @@ static bool attn_mfma_dv(const bf16* q, long q_ld, const bf16* kc, const bf16* v
 #define BFLY_ATT(DVT)                                                                                          \
   attn_window_mfma_kernel<DS, DVT><<<grid, 256, (3 * DVT * 256 + 96) * sizeof(float), s>>>(                    \
       q, q_ld, kc, vc, tables, max_blocks, row_cu, nseq, positions, scale, window, keep_first, sink, out_scale, out, H, \
-      G, fd, nsplit, part, prow)
+      G, fd, nsplit, part, prow, md)
   switch (Dv) {
     case 32: BFLY_ATT(2); break;
     case 64: BFLY_ATT(4); break;
@@ -715,7 +759,8 @@ static bool attn_mfma_dv(const bf16* q, long q_ld, const bf16* kc, const bf16* v
     case 256: BFLY_ATT(16); break;
     default: return false;
   }
-  if (nsplit > 1) attn_split_merge_kernel<<<(unsigned)prow, 64, 0, s>>>(part, prow, nsplit, out_scale, out, Dv);
+  if (nsplit > 1)
+    attn_split_merge_kernel<<<(unsigned)prow, 64, 0, s>>>(part, prow, nsplit, out_scale, out, Dv, md.out_f32);
   return true;
 #undef BFLY_ATT
 }
@@ -723,23 +768,27 @@ static bool attn_mfma_dv(const bf16* q, long q_ld, const bf16* kc, const bf16* v
 bool launch_attn_window_mfma(const void* q, long q_ld, const void* k_cache, const void* v_cache, const int* tables,
                              int max_blocks, const int* row_cu, int nseq, const int* positions, float scale, int window,
                              int keep_first, const float* sink, const float* out_scale, void* out, int T, int H, int G,
-                             int D, int Dv, int block_size, bool fold, float* part, long part_floats, hipStream_t s) {
+                             int D, int Dv, int block_size, bool fold, float* part, long part_floats, hipStream_t s,
+                             const AttnMod& md) {
   if (block_size != 32 || (q_ld & 7) || (reinterpret_cast<uintptr_t>(q) & 15) || (fold && G != 1)) return false;
+  const bool plain = md.chunk == 0 && md.softcap == 0.f && !md.dist_a && md.qt_coef == 0.f && md.maps == 1 && !md.out_f32;
+  if (fold && !plain) return false;        // the folded tile has no score modifiers
   if (T <= 0) return true;
   // few tiles (decoding): several workgroups share a tile's pages, as many as fill the chip, the
   // pages of a row (window and table width bound them) and the scratch allow
   int nsplit = 1;
   {
     const long tiles = (long)(((fold ? T * H : T) + 15) / 16 + nseq) * (fold ? 1 : H);
-    const long pages = std::min<long>((long)window / 32 + 2 + (keep_first + 31) / 32, max_blocks);
+    const long span = md.chunk > 0 ? md.chunk : window;
+    const long pages = std::min<long>(span / 32 + 2 + (keep_first + 31) / 32, max_blocks);
     const long fit = part ? part_floats / ((long)T * H * (Dv + 2)) : 1;
     nsplit = (int)std::max<long>(1, std::min<long>(std::min<long>((256 + tiles - 1) / tiles, pages / 8),
                                                     std::min<long>(fit, 16)));
   }
 #define BFLY_ATTD(DS)                                                                                          \
   return attn_mfma_dv<DS>((const bf16*)q, q_ld, (const bf16*)k_cache, (const bf16*)v_cache, tables, max_blocks, row_cu, \
-                          nseq, positions, scale, window, keep_first, sink, out_scale, (bf16*)out, T, H, G, Dv, fold,    \
-                          nsplit, part, s)
+                          nseq, positions, scale, window, keep_first, sink, out_scale, out, T, H, G, Dv, fold,           \
+                          nsplit, part, s, md)
   switch (D) {
     case 32: BFLY_ATTD(1);
     case 64: BFLY_ATTD(2);
@@ -755,7 +804,7 @@ bool launch_attn_window_mfma(const void* q, long q_ld, const void* k_cache, cons
 void launch_attn_window_paged(const void* q, long q_ld, const void* k_cache, const void* v_cache, const int* tables,
                               int max_blocks, const int* row_seq, int nseq, const int* positions, float scale,
                               int window, int keep_first, const float* sink, const float* out_scale, void* out, int T,
-                              int H, int G, int D, int Dv, int block_size, bool f32, hipStream_t s) {
+                              int H, int G, int D, int Dv, int block_size, bool f32, hipStream_t s, const AttnMod& md) {
   if (T <= 0) return;
   (void)nseq;
   dim3 grid(T, H);
@@ -763,13 +812,13 @@ void launch_attn_window_paged(const void* q, long q_ld, const void* k_cache, con
   if (f32)
     attn_window_paged_kernel<float><<<grid, 64, sm, s>>>((const float*)q, q_ld, (const float*)k_cache,
                                                          (const float*)v_cache, tables, max_blocks, row_seq, positions,
-                                                         scale, window, keep_first, sink, out_scale, (float*)out, H, G,
-                                                         D, Dv, block_size);
+                                                         scale, window, keep_first, sink, out_scale, out, H, G,
+                                                         D, Dv, block_size, md);
   else
     attn_window_paged_kernel<bf16><<<grid, 64, sm, s>>>((const bf16*)q, q_ld, (const bf16*)k_cache,
                                                         (const bf16*)v_cache, tables, max_blocks, row_seq, positions,
-                                                        scale, window, keep_first, sink, out_scale, (bf16*)out, H, G, D,
-                                                        Dv, block_size);
+                                                        scale, window, keep_first, sink, out_scale, out, H, G, D,
+                                                        Dv, block_size, md);
 }
 
 template <typename T>

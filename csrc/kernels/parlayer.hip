@@ -1,0 +1,322 @@
+// Parallel layers with a token shift, per-head normed and half-rotated queries / keys with the
+// paged append, the combination of differential attention maps, and the dense clamped GLU.
+//   par_norm_shift_kernel   x' = x + (ya + yb); both sublayer inputs from one RMS statistic of x'
+//                           (two weights stored around zero); the mixer's input is mixed with the
+//                           previous token's (h + (h_prev - h) shift), whose last value per sequence
+//                           lives in a pooled f32 state
+//   par_final_kernel        the last layer's sum and the output norm of the rows that are asked for
+//   qk_norm_rope_kv_kernel  RMS norm per head, rotation of dimension i with i + n, padded query
+//                           copy, K rows and transposed V rows into the paged caches
+//   diff_combine_kernel     a1 - lambda a2, unit RMS per head, constant factor, sigmoid gate
+//   glu_clamp_kernel        min(g, L) sigmoid(alpha min(g, L)) (clamp(u, +-L) + offset)
+// One workgroup per token row (one wave per head where heads are independent). The residual, the
+// statistics, the state, angles and the combination are f32 whatever the activation type.
+#include <algorithm>
+
+#include "bfly_common.h"
+#include "bfly_parlayer.h"
+
+namespace bfly {
+
+namespace {
+
+// sum of squares of row r of x + (ya + yb), over the workgroup
+template <typename T>
+__device__ __forceinline__ float row_sumsq(const float* __restrict__ x, const T* __restrict__ ya,
+                                           const T* __restrict__ yb, long r, int W, float* red) {
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float v = x[r * W + c];
+    if (ya || yb) v += (ya ? (float)ya[r * W + c] : 0.f) + (yb ? (float)yb[r * W + c] : 0.f);
+    ss = fmaf(v, v, ss);
+  }
+  return block_sum(ss, red);
+}
+
+template <typename T>
+__device__ __forceinline__ float row_val(const float* __restrict__ x, const T* __restrict__ ya,
+                                         const T* __restrict__ yb, long r, int W, int c) {
+  float v = x[r * W + c];
+  if (ya || yb) v += (ya ? (float)ya[r * W + c] : 0.f) + (yb ? (float)yb[r * W + c] : 0.f);
+  return v;
+}
+
+// A row's workgroup recomputes the statistic of row t - 1 (and, for a sequence's first row of the
+// step, of its last row, whose normed value it stores as the new state after it has read the old
+// one): every value is derived from x, ya, yb alone, by the same operations in the same order, so
+// the copies agree bit for bit and no workgroup reads what another one writes.
+template <typename T>
+__global__ __launch_bounds__(256) void par_norm_shift_kernel(const float* __restrict__ x, const T* __restrict__ ya,
+                                                             const T* __restrict__ yb, float* __restrict__ x_out,
+                                                             const float* __restrict__ norm_a,
+                                                             const float* __restrict__ norm_b, float eps, float offset,
+                                                             const float* __restrict__ shift, float* __restrict__ state,
+                                                             const int* __restrict__ state_slots,
+                                                             const int* __restrict__ row_seq,
+                                                             const int* __restrict__ row_cu,
+                                                             const int* __restrict__ positions, T* __restrict__ ha,
+                                                             T* __restrict__ hb, int W) {
+  __shared__ float red[16];
+  const long t = blockIdx.x;
+  const int s = row_seq[t];
+  if (s < 0) {          // padding row of a fixed-shape step
+    for (int c = threadIdx.x; c < W; c += blockDim.x) {
+      ha[t * W + c] = (T)0.f;
+      if (hb) hb[t * W + c] = (T)0.f;
+      if (x_out) x_out[t * W + c] = 0.f;
+    }
+    return;
+  }
+  const float invW = 1.f / (float)W;
+  const float r = 1.f / sqrtf(row_sumsq(x, ya, yb, t, W, red) * invW + eps);
+  const long a = row_cu[s], e = (long)row_cu[s + 1] - 1;
+  const int slot = (shift && state_slots) ? state_slots[s] : -1;
+  // where the previous token's value comes from: 1 the row before, 2 the state, 0 nothing
+  const int src = !shift ? 0 : (t > a ? 1 : ((positions[t] > 0 && slot >= 0) ? 2 : 0));
+  float rp = 0.f;
+  if (src == 1) rp = 1.f / sqrtf(row_sumsq(x, ya, yb, t - 1, W, red) * invW + eps);
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const float v = row_val(x, ya, yb, t, W, c);
+    if (x_out) x_out[t * W + c] = v;
+    const float n = v * r;
+    float h = n * (norm_a[c] + offset);
+    if (hb) hb[t * W + c] = (T)(n * (norm_b[c] + offset));
+    if (shift) {
+      float prev = 0.f;
+      if (src == 1) prev = row_val(x, ya, yb, t - 1, W, c) * rp * (norm_a[c] + offset);
+      else if (src == 2) prev = state[(long)slot * W + c];
+      if (t == a && t == e && slot >= 0) state[(long)slot * W + c] = h;
+      h = h + (prev - h) * shift[c];
+    }
+    ha[t * W + c] = (T)h;
+  }
+  if (shift && t == a && e > a && slot >= 0) {
+    // (this thread read state[slot][c] above, for the same columns c it writes here)
+    const float re = 1.f / sqrtf(row_sumsq(x, ya, yb, e, W, red) * invW + eps);
+    for (int c = threadIdx.x; c < W; c += blockDim.x)
+      state[(long)slot * W + c] = row_val(x, ya, yb, e, W, c) * re * (norm_a[c] + offset);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void par_final_kernel(const float* __restrict__ x, const T* __restrict__ ya,
+                                                        const T* __restrict__ yb, const float* __restrict__ norm_w,
+                                                        float eps, float offset, const long* __restrict__ idx,
+                                                        T* __restrict__ out, int W) {
+  __shared__ float red[16];
+  const long i = blockIdx.x;
+  const long t = idx ? idx[i] : i;
+  const float r = 1.f / sqrtf(row_sumsq(x, ya, yb, t, W, red) / (float)W + eps);
+  for (int c = threadIdx.x; c < W; c += blockDim.x)
+    out[i * W + c] = (T)(row_val(x, ya, yb, t, W, c) * r * (norm_w[c] + offset));
+}
+
+constexpr int kMaxHeadLane = 8;      // head sizes up to 512
+
+// One workgroup per token, one wave per head in turn: the query heads, the key heads, then the
+// value rows. A head is normed in registers (lane l owns dims l, l + 64, ...), staged in LDS so
+// that a rotated dimension finds its partner, and leaves rotated.
+template <typename T>
+__global__ __launch_bounds__(256) void qk_norm_rope_kv_kernel(const T* __restrict__ q, long q_ld, const T* __restrict__ k,
+                                                              long k_ld, const T* __restrict__ v, long v_ld,
+                                                              const float* __restrict__ qn_w,
+                                                              const float* __restrict__ kn_w, float eps,
+                                                              const int* __restrict__ positions,
+                                                              const float* __restrict__ inv_freq, int nrot,
+                                                              const int* __restrict__ slots, T* __restrict__ q_out,
+                                                              T* __restrict__ k_cache, T* __restrict__ v_cache, int Hq,
+                                                              int Gk, int Gv, int D, int Dp, int Dv, int Dvp, int bs) {
+  extern __shared__ float smem[];        // head staging [4][D] | cos [nrot] | sin [nrot]
+  const long t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float* sh = smem + (long)wave * D;
+  float* scos = smem + 4L * D;
+  float* ssin = scos + nrot;
+  const int p = positions[t];
+  // the token's angles once for all heads: f64 product and evaluation of the f32 frequencies
+  for (int f = threadIdx.x; f < nrot; f += blockDim.x) {
+    double sd, cd;
+    sincos((double)p * (double)inv_freq[f], &sd, &cd);
+    scos[f] = (float)cd;
+    ssin[f] = (float)sd;
+  }
+  __syncthreads();
+  const int slot = slots ? slots[t] : -1;
+  const long blk = slot >= 0 ? slot / bs : 0, off = slot >= 0 ? slot % bs : 0;
+  for (int hh = wave; hh < Hq + Gk; hh += 4) {
+    const bool isq = hh < Hq;
+    const int h = isq ? hh : hh - Hq;
+    if (!isq && slot < 0) continue;
+    const T* src = isq ? q + t * q_ld + (long)h * D : k + t * k_ld + (long)h * D;
+    const float* nw = isq ? qn_w : kn_w;
+    float val[kMaxHeadLane];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < kMaxHeadLane; ++i) {
+      const int d = lane + 64 * i;
+      val[i] = d < D ? (float)src[d] : 0.f;
+      ss = fmaf(val[i], val[i], ss);
+    }
+    if (nw) {
+      const float r = 1.f / sqrtf(wave_sum(ss) / (float)D + eps);
+#pragma unroll
+      for (int i = 0; i < kMaxHeadLane; ++i) {
+        const int d = lane + 64 * i;
+        if (d < D) val[i] = val[i] * r * nw[d];
+      }
+    }
+    if (nrot > 0) {
+#pragma unroll
+      for (int i = 0; i < kMaxHeadLane; ++i) {
+        const int d = lane + 64 * i;
+        if (d < D) sh[d] = val[i];
+      }
+      __builtin_amdgcn_wave_barrier();
+      __threadfence_block();
+#pragma unroll
+      for (int i = 0; i < kMaxHeadLane; ++i) {
+        const int d = lane + 64 * i;
+        if (d < 2 * nrot) {
+          const int f = d < nrot ? d : d - nrot;
+          const float c = scos[f], sn = ssin[f];
+          // pair (u, w) = dims (f, f + nrot): u' = u c - w s, w' = w c + u s
+          val[i] = d < nrot ? val[i] * c - sh[d + nrot] * sn : val[i] * c + sh[d - nrot] * sn;
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
+    if (isq) {
+      T* dst = q_out + (t * Hq + h) * Dp;
+#pragma unroll
+      for (int i = 0; i < kMaxHeadLane; ++i) {
+        const int d = lane + 64 * i;
+        if (d < Dp) dst[d] = (T)(d < D ? val[i] : 0.f);
+      }
+    } else {
+      T* dst = k_cache + ((blk * Gk + h) * bs + off) * Dp;
+#pragma unroll
+      for (int i = 0; i < kMaxHeadLane; ++i) {
+        const int d = lane + 64 * i;
+        if (d < D) dst[d] = (T)val[i];
+      }
+    }
+  }
+  if (slot < 0) return;
+  for (int i = threadIdx.x; i < Gv * Dv; i += blockDim.x) {
+    const int g = i / Dv, d = i % Dv;
+    v_cache[((blk * Gv + g) * Dvp + d) * bs + off] = v[t * v_ld + i];
+  }
+}
+
+// One wave per (token, head).
+template <typename T>
+__global__ __launch_bounds__(64) void diff_combine_kernel(const float* __restrict__ a, float lam, float eps,
+                                                          float out_mul, const T* __restrict__ gate, long gate_ld,
+                                                          T* __restrict__ out, int H, int Dv, int Dvp) {
+  const long t = blockIdx.x;
+  const int h = blockIdx.y, lane = threadIdx.x;
+  const float* a1 = a + (t * 2 * H + 2 * h) * Dvp;
+  const float* a2 = a1 + Dvp;
+  float o[kMaxHeadLane];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < kMaxHeadLane; ++i) {
+    const int d = lane + 64 * i;
+    o[i] = d < Dv ? a1[d] - lam * a2[d] : 0.f;
+    ss = fmaf(o[i], o[i], ss);
+  }
+  const float r = out_mul / sqrtf(wave_sum(ss) / (float)Dv + eps);
+#pragma unroll
+  for (int i = 0; i < kMaxHeadLane; ++i) {
+    const int d = lane + 64 * i;
+    if (d < Dv) {
+      float y = o[i] * r;
+      if (gate) y *= 1.f / (1.f + expf(-(float)gate[t * gate_ld + (long)h * Dv + d]));
+      out[(t * H + h) * Dv + d] = (T)y;
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void glu_clamp_kernel(const T* __restrict__ gu, long gu_ld, float limit, float alpha,
+                                                        float up_offset, T* __restrict__ out, long n, int F) {
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+    const long t = i / F;
+    const int f = (int)(i % F);
+    const float g = fminf((float)gu[t * gu_ld + f], limit);
+    const float u = fminf(fmaxf((float)gu[t * gu_ld + F + f], -limit), limit);
+    out[i] = (T)(g / (1.f + expf(-alpha * g)) * (u + up_offset));
+  }
+}
+
+}  // namespace
+
+void launch_par_norm_shift(const float* x, const void* ya, const void* yb, float* x_out, const float* norm_a,
+                           const float* norm_b, float eps, float offset, const float* shift, float* state,
+                           const int* state_slots, const int* row_seq, const int* row_cu, const int* positions,
+                           void* ha, void* hb, int T, int W, bool f32, hipStream_t s) {
+  if (T <= 0) return;
+  if (f32)
+    par_norm_shift_kernel<float><<<T, 256, 0, s>>>(x, (const float*)ya, (const float*)yb, x_out, norm_a, norm_b, eps,
+                                                   offset, shift, state, state_slots, row_seq, row_cu, positions,
+                                                   (float*)ha, (float*)hb, W);
+  else
+    par_norm_shift_kernel<bf16><<<T, 256, 0, s>>>(x, (const bf16*)ya, (const bf16*)yb, x_out, norm_a, norm_b, eps,
+                                                  offset, shift, state, state_slots, row_seq, row_cu, positions,
+                                                  (bf16*)ha, (bf16*)hb, W);
+}
+
+void launch_par_final(const float* x, const void* ya, const void* yb, const float* norm_w, float eps, float offset,
+                      const long* idx, void* out, int R, int W, bool f32, hipStream_t s) {
+  if (R <= 0) return;
+  if (f32)
+    par_final_kernel<float><<<R, 256, 0, s>>>(x, (const float*)ya, (const float*)yb, norm_w, eps, offset, idx,
+                                              (float*)out, W);
+  else
+    par_final_kernel<bf16><<<R, 256, 0, s>>>(x, (const bf16*)ya, (const bf16*)yb, norm_w, eps, offset, idx, (bf16*)out,
+                                             W);
+}
+
+void launch_qk_norm_rope_kv(const void* q, long q_ld, const void* k, long k_ld, const void* v, long v_ld,
+                            const float* qn_w, const float* kn_w, float eps, const int* positions,
+                            const float* inv_freq, int nrot, const int* slots, void* q_out, void* k_cache,
+                            void* v_cache, int T, int Hq, int Gk, int Gv, int D, int Dp, int Dv, int Dvp, int block_size,
+                            bool f32, hipStream_t s) {
+  if (T <= 0) return;
+  const size_t sm = (size_t)(4 * D + 2 * nrot) * sizeof(float);
+  if (f32)
+    qk_norm_rope_kv_kernel<float><<<T, 256, sm, s>>>((const float*)q, q_ld, (const float*)k, k_ld, (const float*)v, v_ld,
+                                                     qn_w, kn_w, eps, positions, inv_freq, nrot, slots, (float*)q_out,
+                                                     (float*)k_cache, (float*)v_cache, Hq, Gk, Gv, D, Dp, Dv, Dvp,
+                                                     block_size);
+  else
+    qk_norm_rope_kv_kernel<bf16><<<T, 256, sm, s>>>((const bf16*)q, q_ld, (const bf16*)k, k_ld, (const bf16*)v, v_ld,
+                                                    qn_w, kn_w, eps, positions, inv_freq, nrot, slots, (bf16*)q_out,
+                                                    (bf16*)k_cache, (bf16*)v_cache, Hq, Gk, Gv, D, Dp, Dv, Dvp,
+                                                    block_size);
+}
+
+void launch_diff_combine(const float* a, float lam, float eps, float out_mul, const void* gate, long gate_ld,
+                         void* out, int T, int H, int Dv, int Dvp, bool f32, hipStream_t s) {
+  if (T <= 0) return;
+  dim3 grid(T, H);
+  if (f32)
+    diff_combine_kernel<float><<<grid, 64, 0, s>>>(a, lam, eps, out_mul, (const float*)gate, gate_ld, (float*)out, H, Dv,
+                                                   Dvp);
+  else
+    diff_combine_kernel<bf16><<<grid, 64, 0, s>>>(a, lam, eps, out_mul, (const bf16*)gate, gate_ld, (bf16*)out, H, Dv,
+                                                  Dvp);
+}
+
+void launch_glu_clamp(const void* gu, long gu_ld, float limit, float alpha, float up_offset, void* out, int T, int F,
+                      bool f32, hipStream_t s) {
+  const long n = (long)T * F;
+  if (n <= 0) return;
+  const unsigned grid = (unsigned)std::min<long>((n + 255) / 256, 65536);
+  if (f32)
+    glu_clamp_kernel<float><<<grid, 256, 0, s>>>((const float*)gu, gu_ld, limit, alpha, up_offset, (float*)out, n, F);
+  else
+    glu_clamp_kernel<bf16><<<grid, 256, 0, s>>>((const bf16*)gu, gu_ld, limit, alpha, up_offset, (bf16*)out, n, F);
+}
+
+}  // namespace bfly
