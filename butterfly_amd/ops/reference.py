@@ -927,8 +927,8 @@ def qk_norm_rope_kv(q, k, v, qn_w, kn_w, eps, positions, inv_freq, slots, k_cach
     inv_freq[i] (f32). q [T, Hq, D] -> q_out [T, Hq, >= D] (zero padded); k [T, Gk, D], v [T, Gv,
     Dv] -> cache rows K [blocks, Gk, BS, >= D], V [blocks, Gv, >= Dv, BS] at slots[t] >= 0."""
     n = inv_freq.numel()
-    a = positions.float()[:, None] * inv_freq.float()[None]
-    c, s = torch.cos(a)[:, None, :], torch.sin(a)[:, None, :]
+    a = positions.double()[:, None] * inv_freq.double()[None]       # the f32 frequencies, f64 product and evaluation
+    c, s = torch.cos(a).float()[:, None, :], torch.sin(a).float()[:, None, :]
 
     def prep(t, w):
         tf = t.float()

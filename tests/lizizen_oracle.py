@@ -140,20 +140,30 @@ def rotate_half(x, base, dims):
     return torch.cat([u * c - v * s, v * c + u * s, x[..., dims:]], -1)
 
 
+def biased_attend(q, k, v, r1, r2, scale, coef, every):
+    """q [n, H, D], k [n, G, D], v [n, G, Dv] -> [n, H, Dv]: causal softmax attention whose scores
+    lose the distance bias, with the query temperature and the sink."""
+    n, H = q.shape[0], q.shape[1]
+    G = k.shape[1]
+    q = q * query_temperature(n, coef, every)[:, None, None]
+    bias = distance_bias(n, r1, r2)
+    mask = causal_mask(n)
+    out = torch.zeros(n, H, v.shape[2], dtype=F64)
+    for hq in range(H):
+        g = hq // (H // G)
+        s = (q[:, hq] @ k[:, g].T) * scale - bias[hq]
+        out[:, hq] = softmax_with_sink(s, mask) @ v[:, g]
+    return out
+
+
 def biased_attention(h, w, p, m):
     n = h.shape[0]
     H, G, D, Dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     q = (h @ w[p + "q"].to(F64).T).view(n, H, D)
     k = (h @ w[p + "k"].to(F64).T).view(n, G, D)
     v = (h @ w[p + "v"].to(F64).T).view(n, G, Dv)
-    q = q * query_temperature(n, m["q_temp"]["coef"], m["q_temp"]["every"])[:, None, None]
-    bias = distance_bias(n, w[p + "r1"], w[p + "r2"])
-    mask = causal_mask(n)
-    out = torch.zeros(n, H, Dv, dtype=F64)
-    for hq in range(H):
-        g = hq // (H // G)
-        s = (q[:, hq] @ k[:, g].T) * m["scale"] - bias[hq]
-        out[:, hq] = softmax_with_sink(s, mask) @ v[:, g]
+    qt = m.get("q_temp") or {"coef": 0.0, "every": 1}
+    out = biased_attend(q, k, v, w[p + "r1"], w[p + "r2"], m["scale"], qt["coef"], qt["every"])
     return out.reshape(n, H * Dv) @ w[p + "o"].to(F64).T
 
 
@@ -162,29 +172,44 @@ def diff_lambda(w, p, diff):
     return float(f("lq1", "lk1") - f("lq2", "lk2") + diff)
 
 
+def normed_rotated(x, nw, eps, base, dims):
+    """x [n, heads, maps, D]: RMS norm per head and map with the shared weight, then the rotation."""
+    n, A, M, D = x.shape
+    x = rms(x, eps) * nw.to(F64)
+    return rotate_half(x.reshape(n, A * M, D), base, dims).view(n, A, M, D) if dims else x
+
+
+def chunk_attend(q, k, v, scale, cap, size):
+    """q [n, H, M, D], k [n, G, M, D], v [n, G, Dv] -> the maps' outputs [n, H, M, Dv]: capped scores,
+    keys of the query's own chunk, ordinary softmax."""
+    n, H, M = q.shape[0], q.shape[1], q.shape[2]
+    G = k.shape[1]
+    mask = chunk_mask(n, size)
+    out = torch.zeros(n, H, M, v.shape[2], dtype=F64)
+    for hq in range(H):
+        g = hq // (H // G)
+        for mp in range(M):
+            s = (q[:, hq, mp] @ k[:, g, mp].T) * scale
+            if cap:
+                s = cap * torch.tanh(s / cap)
+            out[:, hq, mp] = softmax_plain(s, mask) @ v[:, g]
+    return out
+
+
+def combine_maps(a, lam, diff, eps):
+    """a [n, H, 2, Dv] -> [n, H, Dv]: a1 - lambda a2, unit RMS per head, times (1 - diff)."""
+    return rms(a[:, :, 0] - lam * a[:, :, 1], eps) * (1.0 - diff)
+
+
 def diff_attention(h, w, p, m, eps):
     n = h.shape[0]
     H, G, D, Dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    q = (h @ w[p + "q"].to(F64).T).view(n, H, 2, D)
-    k = (h @ w[p + "k"].to(F64).T).view(n, G, 2, D)
+    rot = m.get("rot") or {"base": 1.0, "dims": 0}
+    q = normed_rotated((h @ w[p + "q"].to(F64).T).view(n, H, 2, D), w[p + "q.norm"], eps, rot["base"], rot["dims"])
+    k = normed_rotated((h @ w[p + "k"].to(F64).T).view(n, G, 2, D), w[p + "k.norm"], eps, rot["base"], rot["dims"])
     v = (h @ w[p + "v"].to(F64).T).view(n, G, Dv)
-    q = rms(q, eps) * w[p + "q.norm"].to(F64)
-    k = rms(k, eps) * w[p + "k.norm"].to(F64)
-    q = rotate_half(q.view(n, 2 * H, D), m["rot"]["base"], m["rot"]["dims"]).view(n, H, 2, D)
-    k = rotate_half(k.view(n, 2 * G, D), m["rot"]["base"], m["rot"]["dims"]).view(n, G, 2, D)
-    mask = chunk_mask(n, m["mask"]["size"])
-    lam = diff_lambda(w, p, m["diff"])
-    cap = m["softcap"]
-    out = torch.zeros(n, H, Dv, dtype=F64)
-    for hq in range(H):
-        g = hq // (H // G)
-        a = []
-        for mp in range(2):
-            s = (q[:, hq, mp] @ k[:, g, mp].T) * m["scale"]
-            s = cap * torch.tanh(s / cap)
-            a.append(softmax_plain(s, mask) @ v[:, g])
-        o = a[0] - lam * a[1]
-        out[:, hq] = rms(o, eps) * (1.0 - m["diff"])
+    a = chunk_attend(q, k, v, m["scale"], m.get("softcap") or 0.0, m["mask"]["size"])
+    out = combine_maps(a, diff_lambda(w, p, m["diff"]), m["diff"], eps)
     gate = torch.sigmoid(h @ w[p + "g"].to(F64).T)
     return (out.reshape(n, H * Dv) * gate) @ w[p + "o"].to(F64).T
 
@@ -228,3 +253,11 @@ def forward(cfg, w, tokens, layers_out=None):
         if layers_out is not None:
             layers_out.append(x.clone())
     return offset_norm(x, w["final.norm"], cfg["norm"]["eps"]) @ w["head"].to(F64).T
+
+
+def greedy(cfg, w, prompt, n):
+    """The n tokens greedy decoding appends to the prompt (ties to the lowest id)."""
+    toks = list(prompt)
+    for _ in range(n):
+        toks.append(int(forward(cfg, w, toks)[-1].argmax()))
+    return toks[len(prompt):]
