@@ -92,9 +92,11 @@ def build_parser() -> argparse.ArgumentParser:
                     help="single-stage layouts: host waits for each step's tokens before scheduling the "
                          "next (default: EngineConfig.async_decode, the next step overlaps the host work)")
     ap.add_argument("--out", default=None, help="also write the JSON line here")
-    ap.add_argument("--mixer-family", default="nesizen", choices=["nesizen", "zinesun"],
+    ap.add_argument("--mixer-family", default="nesizen", choices=["nesizen", "zinesun", "lizizen"],
                     help="with --mixer-compare: the heterogeneous family that is timed (nesizen: beside a Mixtral "
-                         "stack; zinesun: latent attention beside a Nesizen stack of plain windowed attention)")
+                         "stack; zinesun: latent attention beside a Nesizen stack of plain windowed attention; "
+                         "lizizen: parallel layers of distance-biased and differential attention with dense GLU "
+                         "feed-forwards beside a Nesizen stack of plain attention with dense feed-forwards)")
     ap.add_argument("--mixer-compare", default=None, metavar="SIZES",
                     help="instead of the headline run: prefill and decode throughput of a Nesizen stack "
                          "(windowed attention, shared keys, gated linear attention, sigmoid MoE) beside a "
@@ -200,6 +202,27 @@ def run_mixer_compare(a) -> int:
                                                  {"type": "attention", "mixer": plain, "mlp": f}
                                                  for f in (dns, moe, dns, moe)]}, name=f"nesizen-attn-{size}")
             pair = (zin, nes2)
+        if a.mixer_family == "lizizen":
+            # distance-biased causal attention with a sink and chunked two-map attention (half the heads,
+            # two maps each, values twice as wide: the same number of score maps and output columns),
+            # dense clamped-GLU feed-forwards, beside plain GQA attention of the same heads (causal where
+            # the biased layers are, a window of the chunk size where the chunked ones are) with dense
+            # feed-forwards of the same parameter count (two matrices of 3/2 the width), one stream
+            bia = {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5, "q_temp": {"coef": 0.1, "every": 256}}
+            dif = {"heads": H // 2, "kv_heads": max(G // 2, 1), "dim": D, "vdim": 2 * D, "scale": D ** -0.5, "diff": 0.6,
+                   "mask": {"size": win}, "rot": {"dims": D // 2, "base": 1e6}, "softcap": 50.0}
+            glu = {"kind": "dense", "ff": dff, "limit": 7.0}
+            liz = ModelConfig.from_lizizen({"architecture": "Lizizen", "vocab": 32000, "width": W, "norm": {"eps": 1e-6},
+                                            "layers": [{"type": t, "mixer": m, "mlp": glu} for t, m in
+                                                       (("attention", bia), ("attention_2", dif)) * 2]},
+                                           name=f"lizizen-{size}")
+            dns = {"kind": "dense", "ff": 3 * dff // 2}
+            nes3 = ModelConfig.from_nesizen({"architecture": "Nesizen", "vocab": 32000, "width": W, "streams": 1,
+                                             "norm": {"eps": 1e-6}, "layers": [
+                                                 {"type": "attention", "mixer": dict(attn, mask={"size": w, "keep_first": 0}),
+                                                  "mlp": dns} for w in (1 << 30, win, 1 << 30, win)]},
+                                            name=f"nesizen-dense-{size}")
+            pair = (liz, nes3)
         for cfg in pair:
             ecfg = EngineConfig(max_batch=B, max_seq_len=P + K + Wm + 8, max_prefill_tokens=8192,
                                 kv_cache_tokens=B * (P + K + Wm + 40), use_graphs=not a.no_graphs,

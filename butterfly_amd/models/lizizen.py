@@ -84,6 +84,13 @@ class LizizenLM(PackedStack):
         # cached head sizes: padded with zeros to sizes the attention's matrix-core form tiles
         self.cache_dims = {sp["index"]: (ops.attn_window_pad(sp["dim"], dtype), ops.attn_window_pad(sp["vdim"], dtype))
                            for sp in self.specs}
+        # feed-forwards whose [gate | up] projection can run on the tuned GEMMs with the fused GLU
+        # epilogue keep its rows (and biases) in alternating 16-row gate / up blocks
+        self.glu_group = {sp["index"]: (ops.SILU_INTERLEAVE if (sp["ffn"] and dtype == torch.bfloat16
+                                                                 and self.device.type == "cuda"
+                                                                 and cfg.hidden_size % 64 == 0
+                                                                 and sp["ffn"]["ff"] % 128 == 0) else 0)
+                          for sp in self.specs}
         self.has_state = bool(self.runs)          # the token shift's previous input, per layer run
         self.state: list = []                     # set by allocate_state (the cache object owns the pool)
         self.layer_probe = None                   # debug hook: f(run, residual [T, W] f32) after every layer run
@@ -131,7 +138,11 @@ class LizizenLM(PackedStack):
             if fs:
                 F = fs["ff"]
                 p[pre + "norm2"] = f(W)
-                p[pre + "gate_up"], p[pre + "gate_up.b"] = z(self._wide(2 * F, W), W), z(self._wide(2 * F, W))
+                if self.glu_group[sp["index"]]:
+                    p[pre + "gate_up"] = z(2 * F, W)
+                    p[pre + "gate_up.b"] = ops.glu_bias_block(z(2 * F), fs["limit"], GLU_ALPHA, GLU_UP_OFFSET)
+                else:
+                    p[pre + "gate_up"], p[pre + "gate_up.b"] = z(self._wide(2 * F, W), W), z(self._wide(2 * F, W))
                 p[pre + "down"], p[pre + "down.b"] = z(self._wide(W, F), F), z(self._wide(W, F))
         p["final.norm"] = f(W)
         p["head"] = z(self.dims.vocab, W)             # rows past the vocabulary stay zero
@@ -188,11 +199,17 @@ class LizizenLM(PackedStack):
                 add(L + "mix.o", p[L + "o"])
             fs = sp["ffn"]
             if fs:
-                F = fs["ff"]
-                add(L + "mlp.gate", p[L + "gate_up"][:F])
-                add(L + "mlp.gate.b", p[L + "gate_up.b"][:F], "small")
-                add(L + "mlp.up", p[L + "gate_up"][F:2 * F])
-                add(L + "mlp.up.b", p[L + "gate_up.b"][F:2 * F], "small")
+                F, grp = fs["ff"], self.glu_group[i]
+                if grp:        # alternating blocks of `grp` gate and up rows
+                    wv, bv = p[L + "gate_up"].view(F // grp, 2, grp, W), p[L + "gate_up.b"][:2 * F].view(F // grp, 2, grp)
+                    for j, n in enumerate(("gate", "up")):
+                        add(L + "mlp." + n, wv[:, j], shape=(F, W), get=lambda t=wv[:, j]: t.reshape(-1, t.shape[-1]))
+                        add(L + "mlp." + n + ".b", bv[:, j], "small", shape=(F,), get=lambda t=bv[:, j]: t.reshape(-1))
+                else:
+                    add(L + "mlp.gate", p[L + "gate_up"][:F])
+                    add(L + "mlp.gate.b", p[L + "gate_up.b"][:F], "small")
+                    add(L + "mlp.up", p[L + "gate_up"][F:2 * F])
+                    add(L + "mlp.up.b", p[L + "gate_up.b"][F:2 * F], "small")
                 add(L + "mlp.down", p[L + "down"][:W])
                 add(L + "mlp.down.b", p[L + "down.b"][:W], "small")
             add(L + "shift", p[L + "shift"], "unit")
@@ -317,7 +334,7 @@ class LizizenLM(PackedStack):
                 ya = self._biased_attention(sp, pre, ha, fb, meta, kv_caches[r])
             else:
                 ya = self._diff_attention(sp, pre, ha, fb, meta, kv_caches[r])
-            yb = self._ffn(sp["ffn"], pre, hb) if sp["ffn"] else None
+            yb = self._ffn(sp, pre, hb) if sp["ffn"] else None
         if self.layer_probe is not None and self.runs:
             self.layer_probe(len(self.runs) - 1, x + (ya.float() + (yb.float() if yb is not None else 0)))
         xf = ops.par_final(x, ya, yb, p["final.norm"], eps, NORM_OFFSET, fb.logits_idx, self.dtype)
@@ -356,9 +373,10 @@ class LizizenLM(PackedStack):
                              z[:, o3:o3 + H * Dv], Dv, self.dtype)
         return ops.linear_act(o, p[pre + "o"])
 
-    def _ffn(self, fs, pre, h):
+    def _ffn(self, sp, pre, h):
+        fs = sp["ffn"]
         p, W, F = self.p, self.cfg.hidden_size, fs["ff"]
-        gu = ops.linear_act(h, p[pre + "gate_up"], bias=p[pre + "gate_up.b"])
-        a = ops.glu_clamp(gu[:, :2 * F], fs["limit"], GLU_ALPHA, GLU_UP_OFFSET)
+        a = ops.linear_glu(h, p[pre + "gate_up"], p[pre + "gate_up.b"], F, fs["limit"], GLU_ALPHA, GLU_UP_OFFSET,
+                           self.glu_group[sp["index"]])
         y = ops.linear_act(a, p[pre + "down"], bias=p[pre + "down.b"])
         return y if y.shape[1] == W else y[:, :W].contiguous()

@@ -18,13 +18,13 @@ from pathlib import Path
 import torch
 
 from . import reference as ref
-from .reference import SILU_INTERLEAVE, interleave_gate_up, rope_tables, split_gate_up  # noqa: F401
+from .reference import SILU_INTERLEAVE, glu_bias_block, interleave_gate_up, rope_tables, split_gate_up  # noqa: F401
 
 _LIB_PATH = Path(__file__).resolve().parent.parent / "_C.so"
 _loaded = False
 _load_error: str | None = None
 
-EPILOGUES = {"none": 0, "bias": 1, "silu": 2}
+EPILOGUES = {"none": 0, "bias": 1, "silu": 2, "glu": 4}
 DECODE_PART_TOKENS = 0   # 0 = pick the context split per call (attn_decode_part_tokens)
 
 
@@ -468,7 +468,10 @@ def pack_w256(w: torch.Tensor) -> torch.Tensor:
 
 def linear(x, w, bias=None, epilogue: str = "none", out=None, defer: bool = False, packed=None):
     """y = x @ w.T (+ bias) with optional fused SwiGLU epilogue ('silu': w rows gate/up
-    interleaved in 16-row groups, output width w.shape[0] // 2). `defer=True` (no bias /
+    interleaved in 16-row groups, output width w.shape[0] // 2) or fused clamped GLU with biases
+    ('glu': the same row layout, `bias` = glu_bias_block(interleaved biases, limit, alpha,
+    up_offset): g sigmoid(alpha g) (u + up_offset), g = min(gate, limit), u = clamp(up,
+    +-limit)). `defer=True` (no bias /
     epilogue): when the plan splits K, return a `Partial` whose reduce the consumer fuses.
     `packed`: the weight's pack_w256 copy: used when the shape's plan has a packed form (decode
     tile plans), else `w`."""
@@ -508,7 +511,7 @@ def linear(x, w, bias=None, epilogue: str = "none", out=None, defer: bool = Fals
     if epilogue == "silu" and bias is not None:
         raise ValueError("bias + silu epilogue not supported")
     M, N = x.shape[0], w.shape[0]
-    nout = N // 2 if epilogue == "silu" else N
+    nout = N // 2 if epilogue in ("silu", "glu") else N
     if out is None:
         out = _empty(M, nout, dtype=x.dtype, device=x.device)
     need = torch.ops.bfly.gemm_workspace_size(M, N, x.shape[1])
@@ -1124,11 +1127,37 @@ def diff_combine(a, lam: float, eps: float, out_mul: float, gate, Dv: int, out_d
     return out
 
 
-def glu_clamp(gu, limit: float, alpha: float, up_offset: float):
-    """gu [T, 2 F] = [gate | up] (rows may be a view): g sigmoid(alpha g) (u + up_offset) with
-    g = min(gate, limit), u = clamp(up, -limit, limit) -> [T, F]."""
+def glu_clamp(gu, limit: float, alpha: float, up_offset: float, group: int = 0):
+    """gu [T, 2 F] = [gate | up] (rows may be a view; group > 0: alternating blocks of `group` gate
+    and up columns, the layout of the GEMMs' fused gate / up epilogues): g sigmoid(alpha g) (u +
+    up_offset) with g = min(gate, limit), u = clamp(up, -limit, limit) -> [T, F]."""
     if not _gpu(gu):
-        return ref.glu_clamp(gu, limit, alpha, up_offset)
+        return ref.glu_clamp(gu, limit, alpha, up_offset, None, group)
     out = _empty(gu.shape[0], gu.shape[1] // 2, dtype=gu.dtype, device=gu.device)
-    torch.ops.bfly.glu_clamp(gu, float(limit), float(alpha), float(up_offset), out)
+    torch.ops.bfly.glu_clamp(gu, float(limit), float(alpha), float(up_offset), int(group), out)
     return out
+
+
+def linear_glu(x, w, bias_block, F: int, limit: float, alpha: float, up_offset: float, group: int = 0):
+    """The clamped-GLU half of a feed-forward: [gate | up] projection with biases and the
+    activation, F columns wide. group == 0: w [2 F (+ padding), K] = [gate rows | up rows] with `bias_block` the
+    matching bias vector; the activation is a pass over the projection. group == SILU_INTERLEAVE:
+    the rows (and biases) alternate in 16-row gate / up blocks and `bias_block` is
+    glu_bias_block(...); bf16 shapes whose GEMM plan has the fused epilogue run as ONE kernel that
+    writes [T, F] only, every other case as projection + pass. Returns [T, rows / 2]."""
+    N = w.shape[0]
+    if group == 0:
+        return glu_clamp(linear_act(x, w, bias=bias_block)[:, :2 * F], limit, alpha, up_offset)
+    if _gpu(x) and _mfma_gemm_ok(x, w, None) and _glu_fused_ok(x.shape[0], N, w.shape[1]):
+        return linear(x, w, bias=bias_block, epilogue="glu")
+    return glu_clamp(linear_act(x, w, bias=bias_block[:N]), limit, alpha, up_offset, group)
+
+
+_glu_ok: dict = {}
+
+
+def _glu_fused_ok(M: int, N: int, K: int) -> bool:
+    ok = _glu_ok.get((M, N, K))
+    if ok is None:
+        ok = _glu_ok[(M, N, K)] = torch.ops.bfly.gemm_check(M, N, K, EPILOGUES["glu"]) == 0
+    return ok

@@ -314,8 +314,22 @@ def topkp_threshold(logits, temps, top_k, top_p, reduce_sum=None, reduce_max=Non
     return out
 
 
+def glu_bias_block(bias, limit, alpha, up_offset):
+    """The fused clamped-GLU epilogue's block: N bias values (bf16, interleaved like the weight's
+    rows) followed by {limit, alpha, up_offset} as three f32 values in six bf16 slots."""
+    blk = torch.zeros(bias.numel() + 6, dtype=torch.bfloat16, device=bias.device)
+    blk[:bias.numel()] = bias.to(torch.bfloat16)
+    blk[bias.numel():].view(torch.float32).copy_(torch.tensor([limit, alpha, up_offset], dtype=torch.float32))
+    return blk
+
+
 def linear(x, w, bias=None, epilogue="none", out=None):
     y = x.float() @ w.float().t()
+    if epilogue == "glu":       # bias = glu_bias_block(...): clamped GLU on interleaved gate / up rows
+        N = w.shape[0]
+        lim, alpha, off = bias[N:].view(torch.float32).tolist()
+        y = glu_clamp(y + bias[:N].float(), lim, alpha, off, torch.float32, SILU_INTERLEAVE)
+        bias = None
     if bias is not None:
         y = y + bias.float()
     if epilogue == "silu":
@@ -965,9 +979,10 @@ def diff_combine(a, lam, eps, out_mul, gate, Dv, out_dtype):
     return o.to(out_dtype)
 
 
-def glu_clamp(gu, limit, alpha, up_offset, out_dtype=None):
-    """gu [T, 2 F] = [gate | up]: min(g, limit) sigmoid(alpha min(g, limit)) (clamp(u, +-limit) + up_offset)."""
-    F = gu.shape[1] // 2
-    g = gu[:, :F].float().clamp(max=limit)
-    u = gu[:, F:].float().clamp(min=-limit, max=limit)
+def glu_clamp(gu, limit, alpha, up_offset, out_dtype=None, group=0):
+    """gu [T, 2 F] = [gate | up] (group > 0: alternating blocks of `group` gate and up columns):
+    min(g, limit) sigmoid(alpha min(g, limit)) (clamp(u, +-limit) + up_offset)."""
+    g, u = split_gate_up(gu, group)
+    g = g.float().clamp(max=limit)
+    u = u.float().clamp(min=-limit, max=limit)
     return (g * torch.sigmoid(alpha * g) * (u + up_offset)).to(out_dtype or gu.dtype)

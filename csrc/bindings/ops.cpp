@@ -358,11 +358,17 @@ void gemm(const Tensor& x, const Tensor& w, Tensor& out, const c10::optional<Ten
   TORCH_CHECK(x.stride(0) % 8 == 0 && w.stride(0) % 8 == 0, "gemm: row strides % 8");
   TORCH_CHECK(K % 64 == 0, "gemm: K must be a multiple of 64, got ", K);
   TORCH_CHECK(N % 128 == 0, "gemm: N must be a multiple of 128, got ", N);
-  const int nout = epilogue == bfly::EPI_SILU ? N / 2 : N;
+  const int nout = bfly::epi_halves((int)epilogue) ? N / 2 : N;
   TORCH_CHECK(out.size(0) == M && out.size(1) == nout, "gemm: out shape");
   const bfly::bf16* bp = nullptr;
   if (epilogue == bfly::EPI_BIAS) {
     TORCH_CHECK(bias.has_value() && bias->numel() == N, "gemm: bias required");
+    CHECK_BF16(*bias);
+    bp = bf(*bias);
+  } else if (epilogue == bfly::EPI_GLU) {
+    // N interleaved bias values, then {limit, alpha, offset} as three f32
+    TORCH_CHECK(bias.has_value() && bias->numel() == N + bfly::kGluBlockTail && bias->is_contiguous() &&
+                    reinterpret_cast<uintptr_t>(bias->data_ptr()) % 4 == 0, "gemm: the GLU epilogue needs its bias block");
     CHECK_BF16(*bias);
     bp = bf(*bias);
   }

@@ -145,13 +145,14 @@ void diff_combine(const Tensor& a, double lam, double eps, double out_mul, const
                             (int)H, (int)Dv, (int)Dvp, is_f32(out), cur_stream());
 }
 
-void glu_clamp(const Tensor& gu, double limit, double alpha, double up_offset, Tensor& out) {
+void glu_clamp(const Tensor& gu, double limit, double alpha, double up_offset, int64_t group, Tensor& out) {
   CHK_GPU(gu); CHK_SAME(gu, out);
   TORCH_CHECK(gu.dim() == 2 && gu.stride(1) == 1 && gu.size(1) % 2 == 0 && out.dim() == 2 && out.is_contiguous(), "glu_clamp: layouts");
   const int64_t T = gu.size(0), F = gu.size(1) / 2;
   TORCH_CHECK(out.size(0) == T && out.size(1) == F, "glu_clamp: out [T, F]");
+  TORCH_CHECK(group >= 0 && (group == 0 || F % group == 0), "glu_clamp: the interleave group must divide F");
   bfly::launch_glu_clamp(gu.data_ptr(), gu.stride(0), (float)limit, (float)alpha, (float)up_offset, out.data_ptr(), (int)T,
-                         (int)F, is_f32(gu), cur_stream());
+                         (int)F, (int)group, is_f32(gu), cur_stream());
 }
 
 }  // namespace
@@ -165,7 +166,7 @@ TORCH_LIBRARY_FRAGMENT(bfly, m) {
   m.def("qk_norm_rope_kv(Tensor q, Tensor k, Tensor v, Tensor? qn_w, Tensor? kn_w, float eps, Tensor positions, "
         "Tensor inv_freq, Tensor slots, Tensor(a!) k_cache, Tensor(b!) v_cache, Tensor(c!) q_out) -> ()");
   m.def("diff_combine(Tensor a, float lam, float eps, float out_mul, Tensor? gate, int Dv, Tensor(a!) out) -> ()");
-  m.def("glu_clamp(Tensor gu, float limit, float alpha, float up_offset, Tensor(a!) out) -> ()");
+  m.def("glu_clamp(Tensor gu, float limit, float alpha, float up_offset, int group, Tensor(a!) out) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(bfly, CUDA, m) {

@@ -11,7 +11,15 @@ typedef __bf16 bf16;
 
 // EPI_SILU_GATE: the SwiGLU epilogue followed by the MoE dense decode path's routing weight
 // (what moe_gate_scale did as a separate pass): see RowScale::gate.
-enum GemmEpilogue { EPI_NONE = 0, EPI_BIAS = 1, EPI_SILU = 2, EPI_SILU_GATE = 3 };
+// EPI_GLU: a clamped GLU with biases on gate / up rows interleaved as for EPI_SILU:
+//   Y[M, N/2] = g sigmoid(alpha g) (u + offset), g = min(gate + b_gate, limit), u = clamp(up + b_up, +-limit).
+//   `bias` then points at the epilogue's block: N bias values (bf16, interleaved like the rows)
+//   followed by the three f32 values {limit, alpha, offset} (N is even, so they are 4-byte
+//   aligned): the parameters travel with the bias, the kernels' signatures stay as they are.
+enum GemmEpilogue { EPI_NONE = 0, EPI_BIAS = 1, EPI_SILU = 2, EPI_SILU_GATE = 3, EPI_GLU = 4 };
+constexpr int kGluBlockTail = 6;      // bf16 slots of the three f32 parameters after the N bias values
+// epilogues that pair gate / up 16-row groups and write N / 2 columns
+inline bool epi_halves(int epi) { return epi == EPI_SILU || epi == EPI_GLU; }
 
 // Per-row output scales of the tile / decode-ring / mid-M epilogues.
 // RMSNorm: the X rows are un-normalised RMSNorm inputs (x * g); row m is multiplied by

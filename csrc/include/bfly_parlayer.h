@@ -35,8 +35,10 @@ void launch_qk_norm_rope_kv(const void* q, long q_ld, const void* k, long k_ld, 
 // o / rms(o) * out_mul * sigmoid(gate[t, h * Dv + d]) (gate nullable) -> out [T, H * Dv]. Dv <= 512.
 void launch_diff_combine(const float* a, float lam, float eps, float out_mul, const void* gate, long gate_ld,
                          void* out, int T, int H, int Dv, int Dvp, bool f32, hipStream_t s);
-// out[t, f] = g sigmoid(alpha g) (u + up_offset), g = min(gu[t, f], limit), u = clamp(gu[t, F + f], +-limit)
+// out[t, f] = g sigmoid(alpha g) (u + up_offset), g = min(gate, limit), u = clamp(up, +-limit); gate / up of
+// column f are gu[t, f] and gu[t, F + f] (group == 0), or lie in alternating blocks of `group` columns
+// (gate block, up block, ...: the row layout of the GEMMs' fused gate / up epilogues)
 void launch_glu_clamp(const void* gu, long gu_ld, float limit, float alpha, float up_offset, void* out, int T, int F,
-                      bool f32, hipStream_t s);
+                      int group, bool f32, hipStream_t s);
 
 }  // namespace bfly

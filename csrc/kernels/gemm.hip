@@ -7,6 +7,9 @@
 //   EPI_BIAS  : Y = acc + bias[n]
 //   EPI_SILU  : W's rows are gate/up interleaved in 16-row groups (g0 u0 g1 u1 ...);
 //               Y[M, N/2] = silu(gate) * up  (the SwiGLU FFN's first half in one kernel)
+//   EPI_GLU   : the same row layout; Y[M, N/2] = g sigmoid(alpha g) (u + offset) with g = min(gate
+//               + bias, limit), u = clamp(up + bias, +-limit); bias and the three constants come
+//               in one block (bfly_kernels.h)
 //
 // Two kernels, picked by M on the host:
 //  * gemm_skinny (M <= 64, decode): weight-streaming. Each wave streams 16*NT rows of W
@@ -48,6 +51,20 @@ __device__ __forceinline__ void store_out(bf16* out, long ldo, int m, int n, flo
   out[(long)m * ldo + n] = f2bf(v);
 }
 
+// EPI_GLU: the constants behind the N bias values, and the activation of a (gate, up) pair.
+struct GluPar {
+  float limit, alpha, offset;
+};
+__device__ __forceinline__ GluPar glu_par(const bf16* bias, int N) {
+  const float* f = reinterpret_cast<const float*>(bias + N);
+  return GluPar{f[0], f[1], f[2]};
+}
+__device__ __forceinline__ float glu_clamped(float g, float u, const GluPar& p) {
+  g = fminf(g, p.limit);
+  u = fminf(fmaxf(u, -p.limit), p.limit);
+  return g / (1.f + __expf(-p.alpha * g)) * (u + p.offset);
+}
+
 // Four consecutive output columns of one row (the tile / decode-ring accumulators hold 4
 // consecutive n per lane: W is their MFMA A operand). 8-B store when the row start allows it.
 __device__ __forceinline__ void store_out4(bf16* out, long ldo, int m, int n, f32x4 v, bool vec) {
@@ -82,13 +99,14 @@ __device__ __forceinline__ void store_slab4(__amdgpu_buffer_rsrc_t r, int off, f
 __global__ void gemm_splitk_reduce_kernel(const float* __restrict__ part, int SK, int M, int N,
                                           int epi, const bf16* __restrict__ bias,
                                           bf16* __restrict__ out, long ldo) {
-  const int nout = epi == EPI_SILU ? N / 2 : N;
+  const bool halves = epi == EPI_SILU || epi == EPI_GLU;
+  const int nout = halves ? N / 2 : N;
   const long total = (long)M * nout;
   const long slab = (long)M * N;
   for (long e = blockIdx.x * (long)blockDim.x + threadIdx.x; e < total;
        e += (long)gridDim.x * blockDim.x) {
     const int m = (int)(e / nout), f = (int)(e % nout);
-    if (epi == EPI_SILU) {
+    if (halves) {
       const int g = f >> 4, w = f & 15;
       const long gi = (long)m * N + g * 32 + w, ui = gi + 16;
       float gs = 0.f, us = 0.f;
@@ -96,7 +114,10 @@ __global__ void gemm_splitk_reduce_kernel(const float* __restrict__ part, int SK
         gs += part[s * slab + gi];
         us += part[s * slab + ui];
       }
-      store_out(out, ldo, m, f, silu(gs) * us);
+      if (epi == EPI_GLU)
+        store_out(out, ldo, m, f, glu_clamped(gs + bf2f(bias[g * 32 + w]), us + bf2f(bias[g * 32 + w + 16]), glu_par(bias, N)));
+      else
+        store_out(out, ldo, m, f, silu(gs) * us);
     } else {
       const long i = (long)m * N + f;
       float acc = 0.f;
@@ -202,7 +223,7 @@ gemm_skinny_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict_
       for (int i = 0; i < 4; ++i) red[wid * E + ((t * MT + mt) * 4 + i) * 64 + lane] = acc[t][mt][i];
   __syncthreads();
 
-  const bool silu_epi = epi == EPI_SILU;
+  const bool silu_epi = epi == EPI_SILU || epi == EPI_GLU;
   for (int idx = threadIdx.x; idx < WN * E; idx += kSkThreads) {
     const int vn = idx / E, e = idx % E;
     const int l = e & 63, i = (e >> 6) & 3, tm = e >> 8;
@@ -223,7 +244,10 @@ gemm_skinny_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict_
 #pragma unroll
       for (int k = 0; k < WK; ++k) u += red[(vn * WK + k) * E + eu];
       const int f = nw0 / 2 + 16 * (t / 2) + (l >> 4) * 4 + i;
-      store_out(out, ldo, m, f, silu(v) * u);
+      if (epi == EPI_GLU)
+        store_out(out, ldo, m, f, glu_clamped(v + bf2f(bias[n]), u + bf2f(bias[n + 16]), glu_par(bias, N)));
+      else
+        store_out(out, ldo, m, f, silu(v) * u);
     } else {
       store_out(out, ldo, m, n, epi == EPI_BIAS ? v + bf2f(bias[n]) : v);
     }
@@ -337,12 +361,19 @@ __device__ __forceinline__ void tile_epilogue(const f32x4 (&acc)[TI][TJ], int mw
       const int n = nw + 16 * j + lc;
       if (pslab) {
         store_slab4(rs, ((m - m0) * N + n) * 4, acc[i][j] * sc[i]);
-      } else if (epi == EPI_SILU || epi == EPI_SILU_GATE) {
+      } else if (epi == EPI_SILU || epi == EPI_SILU_GATE || epi == EPI_GLU) {
         if constexpr (TJ % 2 == 0) {   // gate/up 16-row groups pair up inside the wave
           if (j & 1) continue;
           f32x4 h;
+          if (epi == EPI_GLU) {
+            const GluPar gp = glu_par(bias, N);
 #pragma unroll
-          for (int r = 0; r < 4; ++r) h[r] = silu(acc[i][j][r] * sc[i]) * (acc[i][j + 1][r] * sc[i]);
+            for (int r = 0; r < 4; ++r)
+              h[r] = glu_clamped(acc[i][j][r] * sc[i] + bf2f(bias[n + r]), acc[i][j + 1][r] * sc[i] + bf2f(bias[n + 16 + r]), gp);
+          } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) h[r] = silu(acc[i][j][r] * sc[i]) * (acc[i][j + 1][r] * sc[i]);
+          }
           const int f = nw / 2 + 16 * (j / 2) + lc;
           if (epi == EPI_SILU_GATE) {   // the 4 columns share an expert (gF % 16 == 0)
             const float g = rsc.gate[(long)m * rsc.gld + rsc.ge0 + f / rsc.gF];
@@ -1733,7 +1764,7 @@ static int run_plan(const GemmPlan& p, const bf16* X, long ldx, const bf16* W, l
     // mid-M 8-wave staggered GEMM: plan {5, SW (weight ring), SX (activation ring; 0 = SW), 0,
     // BM, BN, sk}
     if (N % p.bn != 0 || K % kBK != 0 || K / kBK < p.sk) return -1;
-    if (epi == EPI_SILU && p.bn * p.bm / 512 % 32 != 0) return -1;
+    if (epi_halves(epi) && p.bn * p.bm / 512 % 32 != 0) return -1;
     const int sx = p.nt > 0 ? p.nt : p.mt;
     bool done = false;
 #define MID_CASE(BM_, BN_, SX_, SW_)                                                              \
@@ -1752,7 +1783,7 @@ static int run_plan(const GemmPlan& p, const bf16* X, long ldx, const bf16* W, l
     // decode ring GEMM: plan {3, SW (weight ring depth), waves, waves along M, BM, BN, sk}
     if (N % p.bn != 0 || K % kBK != 0 || K / kBK < p.sk * 2) return -1;
     const int nwn = p.wk > 0 ? p.nt / p.wk : 0;
-    if (epi == EPI_SILU && (nwn <= 0 || (p.bn / nwn) % 32 != 0)) return -1;
+    if (epi_halves(epi) && (nwn <= 0 || (p.bn / nwn) % 32 != 0)) return -1;
     bool done = false;
 #define DEC_CASE(BM_, BN_, NWM_, NWN_, SW_)                                                      \
   if (!done && p.bm == BM_ && p.bn == BN_ && p.wk == NWM_ && p.nt == NWM_ * NWN_ && p.mt == SW_) { \
@@ -1769,7 +1800,7 @@ static int run_plan(const GemmPlan& p, const bf16* X, long ldx, const bf16* W, l
   } else if (p.kind == 0) {
     if (K % 128 != 0 || M > 16 * p.mt) return -1;
     if (N % (16 * p.nt * (4 / p.wk)) != 0) return -1;
-    if (epi == EPI_SILU && p.nt % 2 != 0) return -1;
+    if (epi_halves(epi) && p.nt % 2 != 0) return -1;
     if (p.sk > 1 && N / (16 * p.nt * (4 / p.wk)) > kSplitCounters) return -1;
     bool done = false;
 #define SK_CASE(MT_, NT_, WK_)                                                                   \
@@ -1826,7 +1857,7 @@ static int run_plan(const GemmPlan& p, const bf16* X, long ldx, const bf16* W, l
     if (!done) return -2;
   }
   if (p.sk > 1 && !dry && !defer) {
-    const int nout = epi == EPI_SILU ? N / 2 : N;
+    const int nout = epi_halves(epi) ? N / 2 : N;
     long total = (long)M * nout;
     int grid = (int)((total + 255) / 256);
     if (grid > 4096) grid = 4096;

@@ -76,10 +76,16 @@ __device__ __forceinline__ float attn_row_scale(int p, float scale, const AttnMo
   if (md.qt_coef == 0.f) return scale;
   return scale * (1.f + md.qt_coef * logf((float)((p + 1) / md.qt_every) + 1.f));
 }
+// FAST (the bf16 matrix-core form): hardware exp / log / reciprocal; the generic form, which also
+// serves true-f32 runs, keeps the precise functions.
+template <bool FAST>
 __device__ __forceinline__ float attn_score(float dot, float rscale, int dist, float da, float db, const AttnMod& md) {
   float sc = dot * rscale;
-  if (md.softcap > 0.f) sc = md.softcap * tanhf(sc / md.softcap);
-  if (md.dist_a) sc -= da * log1pf(db * (float)dist);
+  if (md.softcap > 0.f) {
+    if (FAST) sc = md.softcap * (1.f - __fdividef(2.f, __expf(2.f * __fdividef(sc, md.softcap)) + 1.f));
+    else sc = md.softcap * tanhf(sc / md.softcap);
+  }
+  if (md.dist_a) sc -= da * (FAST ? __logf(1.f + db * (float)dist) : log1pf(db * (float)dist));
   return sc;
 }
 
@@ -137,7 +143,7 @@ __global__ __launch_bounds__(64) void attn_window_paged_kernel(const T* __restri
       const T* kr = k_cache + ((blk * Gk + gk) * bs + (j % bs)) * D;
       float a = 0.f;
       for (int d = 0; d < D; ++d) a = fmaf(sq[d], (float)kr[d], a);
-      sc = attn_score(a, rscale, p - j, da, db, md);
+      sc = attn_score<false>(a, rscale, p - j, da, db, md);
     }
     const float mn = fmaxf(m, wave_max(sc));
     const float pe = i < total ? expf(sc - mn) : 0.f;
@@ -288,7 +294,7 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __res
       for (int i = 0; i < 4; ++i) {
         const int j = pg * BS + 16 * kh + 4 * gg + i;
         const bool ok = j <= p && (j >= plo || j < keep_first);
-        sc[4 * kh + i] = ok ? attn_score(st[kh][i], rscale, p - j, da, db, md) : -INFINITY;
+        sc[4 * kh + i] = ok ? attn_score<true>(st[kh][i], rscale, p - j, da, db, md) : -INFINITY;
         mx = fmaxf(mx, sc[4 * kh + i]);
       }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));

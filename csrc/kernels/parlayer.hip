@@ -98,6 +98,121 @@ __global__ __launch_bounds__(256) void par_norm_shift_kernel(const float* __rest
   }
 }
 
+// Four consecutive elements of a row as floats.
+__device__ __forceinline__ f32x4 ld4(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
+__device__ __forceinline__ f32x4 ld4(const bf16* p) {
+  const bf16x4 v = *reinterpret_cast<const bf16x4*>(p);
+  return f32x4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+}
+__device__ __forceinline__ void st4(float* p, f32x4 v) { *reinterpret_cast<f32x4*>(p) = v; }
+__device__ __forceinline__ void st4(bf16* p, f32x4 v) {
+  *reinterpret_cast<bf16x4*>(p) = bf16x4{(bf16)v[0], (bf16)v[1], (bf16)v[2], (bf16)v[3]};
+}
+
+// Row r of x + (ya + yb) into registers, VPT groups of four columns per thread (group k of thread
+// i: columns 4 (i + 256 k) ...); returns the row's sum of squares over the workgroup. Every user
+// sums in this one order, so the copies of a row's statistic agree bit for bit.
+template <typename T, int VPT>
+__device__ __forceinline__ float row_load4(const float* __restrict__ x, const T* __restrict__ ya,
+                                           const T* __restrict__ yb, long r, int W, f32x4 (&v)[VPT], float* red) {
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    const int c = 4 * (threadIdx.x + 256 * k);
+    v[k] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (c < W) {
+      v[k] = ld4(x + r * W + c);
+      if (ya || yb) {
+        const f32x4 a = ya ? ld4(ya + r * W + c) : f32x4{0.f, 0.f, 0.f, 0.f};
+        const f32x4 b = yb ? ld4(yb + r * W + c) : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[k][i] += a[i] + b[i];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ss = fmaf(v[k][i], v[k][i], ss);
+  }
+  return block_sum(ss, red);
+}
+
+// par_norm_shift_kernel for rows of W % 4 == 0, W <= 1024 VPT columns: each row is read once into
+// registers with 16-byte (f32) / 8-byte (bf16) accesses.
+template <typename T, int VPT>
+__global__ __launch_bounds__(256) void par_norm_shift_vec_kernel(
+    const float* __restrict__ x, const T* __restrict__ ya, const T* __restrict__ yb, float* __restrict__ x_out,
+    const float* __restrict__ norm_a, const float* __restrict__ norm_b, float eps, float offset,
+    const float* __restrict__ shift, float* __restrict__ state, const int* __restrict__ state_slots,
+    const int* __restrict__ row_seq, const int* __restrict__ row_cu, const int* __restrict__ positions,
+    T* __restrict__ ha, T* __restrict__ hb, int W) {
+  __shared__ float red[16];
+  const long t = blockIdx.x;
+  const int s = row_seq[t];
+  const f32x4 zero = f32x4{0.f, 0.f, 0.f, 0.f};
+  if (s < 0) {          // padding row of a fixed-shape step
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      const int c = 4 * (threadIdx.x + 256 * k);
+      if (c >= W) continue;
+      st4(ha + t * W + c, zero);
+      if (hb) st4(hb + t * W + c, zero);
+      if (x_out) st4(x_out + t * W + c, zero);
+    }
+    return;
+  }
+  const float invW = 1.f / (float)W;
+  f32x4 v[VPT], pv[VPT];
+  const float r = 1.f / sqrtf(row_load4<T, VPT>(x, ya, yb, t, W, v, red) * invW + eps);
+  const long a = row_cu[s], e = (long)row_cu[s + 1] - 1;
+  const int slot = (shift && state_slots) ? state_slots[s] : -1;
+  const int src = !shift ? 0 : (t > a ? 1 : ((positions[t] > 0 && slot >= 0) ? 2 : 0));
+  float rp = 0.f;
+  if (src == 1) rp = 1.f / sqrtf(row_load4<T, VPT>(x, ya, yb, t - 1, W, pv, red) * invW + eps);
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    const int c = 4 * (threadIdx.x + 256 * k);
+    if (c >= W) continue;
+    if (x_out) st4(x_out + t * W + c, v[k]);
+    const f32x4 wa = ld4(norm_a + c);
+    f32x4 h, o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) h[i] = v[k][i] * r * (wa[i] + offset);
+    if (hb) {
+      const f32x4 wb = ld4(norm_b + c);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[i] = v[k][i] * r * (wb[i] + offset);
+      st4(hb + t * W + c, o);
+    }
+    if (shift) {
+      f32x4 prev = zero;
+      if (src == 1) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) prev[i] = pv[k][i] * rp * (wa[i] + offset);
+      } else if (src == 2) {
+        prev = ld4(state + (long)slot * W + c);
+      }
+      if (t == a && t == e && slot >= 0) st4(state + (long)slot * W + c, h);
+      const f32x4 sh = ld4(shift + c);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) h[i] = h[i] + (prev[i] - h[i]) * sh[i];
+    }
+    st4(ha + t * W + c, h);
+  }
+  if (shift && t == a && e > a && slot >= 0) {
+    // (this thread read state[slot] above, for the same columns it writes here)
+    const float re = 1.f / sqrtf(row_load4<T, VPT>(x, ya, yb, e, W, pv, red) * invW + eps);
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      const int c = 4 * (threadIdx.x + 256 * k);
+      if (c >= W) continue;
+      const f32x4 wa = ld4(norm_a + c);
+      f32x4 h;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) h[i] = pv[k][i] * re * (wa[i] + offset);
+      st4(state + (long)slot * W + c, h);
+    }
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void par_final_kernel(const float* __restrict__ x, const T* __restrict__ ya,
                                                         const T* __restrict__ yb, const float* __restrict__ norm_w,
@@ -113,9 +228,10 @@ __global__ __launch_bounds__(256) void par_final_kernel(const float* __restrict_
 
 constexpr int kMaxHeadLane = 8;      // head sizes up to 512
 
-// One workgroup per token, one wave per head in turn: the query heads, the key heads, then the
-// value rows. A head is normed in registers (lane l owns dims l, l + 64, ...), staged in LDS so
-// that a rotated dimension finds its partner, and leaves rotated.
+// One workgroup per (token, group of four heads), one wave per head: the query heads, then the key
+// heads; the workgroups of a token share the copy of its value rows. A head is normed in registers
+// (lane l owns dims l, l + 64, ...), staged in LDS so that a rotated dimension finds its partner,
+// and leaves rotated.
 template <typename T>
 __global__ __launch_bounds__(256) void qk_norm_rope_kv_kernel(const T* __restrict__ q, long q_ld, const T* __restrict__ k,
                                                               long k_ld, const T* __restrict__ v, long v_ld,
@@ -143,10 +259,10 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_kernel(const T* __restric
   __syncthreads();
   const int slot = slots ? slots[t] : -1;
   const long blk = slot >= 0 ? slot / bs : 0, off = slot >= 0 ? slot % bs : 0;
-  for (int hh = wave; hh < Hq + Gk; hh += 4) {
+  const int hh = 4 * blockIdx.y + wave;
+  if (hh < Hq + Gk && (hh < Hq || slot >= 0)) {
     const bool isq = hh < Hq;
     const int h = isq ? hh : hh - Hq;
-    if (!isq && slot < 0) continue;
     const T* src = isq ? q + t * q_ld + (long)h * D : k + t * k_ld + (long)h * D;
     const float* nw = isq ? qn_w : kn_w;
     float val[kMaxHeadLane];
@@ -202,7 +318,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_kernel(const T* __restric
     }
   }
   if (slot < 0) return;
-  for (int i = threadIdx.x; i < Gv * Dv; i += blockDim.x) {
+  for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < Gv * Dv; i += gridDim.y * blockDim.x) {
     const int g = i / Dv, d = i % Dv;
     v_cache[((blk * Gv + g) * Dvp + d) * bs + off] = v[t * v_ld + i];
   }
@@ -239,12 +355,15 @@ __global__ __launch_bounds__(64) void diff_combine_kernel(const float* __restric
 
 template <typename T>
 __global__ __launch_bounds__(256) void glu_clamp_kernel(const T* __restrict__ gu, long gu_ld, float limit, float alpha,
-                                                        float up_offset, T* __restrict__ out, long n, int F) {
+                                                        float up_offset, T* __restrict__ out, long n, int F,
+                                                        int group) {
   for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
     const long t = i / F;
     const int f = (int)(i % F);
-    const float g = fminf((float)gu[t * gu_ld + f], limit);
-    const float u = fminf(fmaxf((float)gu[t * gu_ld + F + f], -limit), limit);
+    const int cg = group > 0 ? (f / group) * 2 * group + f % group : f;       // the gate's column
+    const int cu = group > 0 ? cg + group : F + f;
+    const float g = fminf((float)gu[t * gu_ld + cg], limit);
+    const float u = fminf(fmaxf((float)gu[t * gu_ld + cu], -limit), limit);
     out[i] = (T)(g / (1.f + expf(-alpha * g)) * (u + up_offset));
   }
 }
@@ -256,6 +375,24 @@ void launch_par_norm_shift(const float* x, const void* ya, const void* yb, float
                            const int* state_slots, const int* row_seq, const int* row_cu, const int* positions,
                            void* ha, void* hb, int T, int W, bool f32, hipStream_t s) {
   if (T <= 0) return;
+  const auto al = [](const void* p, size_t n) { return (reinterpret_cast<uintptr_t>(p) & (n - 1)) == 0; };
+  const size_t ea = f32 ? 16 : 8;
+  if (W % 4 == 0 && W <= 8192 && al(x, 16) && al(x_out, 16) && al(norm_a, 16) && al(norm_b, 16) && al(shift, 16) &&
+      al(state, 16) && al(ya, ea) && al(yb, ea) && al(ha, ea) && al(hb, ea)) {
+#define BFLY_PNS(TT, V)                                                                                          \
+  par_norm_shift_vec_kernel<TT, V><<<T, 256, 0, s>>>(x, (const TT*)ya, (const TT*)yb, x_out, norm_a, norm_b, eps,   \
+                                                    offset, shift, state, state_slots, row_seq, row_cu, positions, \
+                                                    (TT*)ha, (TT*)hb, W)
+#define BFLY_PNSV(TT)                \
+  if (W <= 1024) BFLY_PNS(TT, 1);    \
+  else if (W <= 2048) BFLY_PNS(TT, 2); \
+  else if (W <= 4096) BFLY_PNS(TT, 4); \
+  else BFLY_PNS(TT, 8)
+    if (f32) { BFLY_PNSV(float); } else { BFLY_PNSV(bf16); }
+#undef BFLY_PNSV
+#undef BFLY_PNS
+    return;
+  }
   if (f32)
     par_norm_shift_kernel<float><<<T, 256, 0, s>>>(x, (const float*)ya, (const float*)yb, x_out, norm_a, norm_b, eps,
                                                    offset, shift, state, state_slots, row_seq, row_cu, positions,
@@ -284,13 +421,14 @@ void launch_qk_norm_rope_kv(const void* q, long q_ld, const void* k, long k_ld, 
                             bool f32, hipStream_t s) {
   if (T <= 0) return;
   const size_t sm = (size_t)(4 * D + 2 * nrot) * sizeof(float);
+  const dim3 grid(T, (Hq + Gk + 3) / 4);
   if (f32)
-    qk_norm_rope_kv_kernel<float><<<T, 256, sm, s>>>((const float*)q, q_ld, (const float*)k, k_ld, (const float*)v, v_ld,
+    qk_norm_rope_kv_kernel<float><<<grid, 256, sm, s>>>((const float*)q, q_ld, (const float*)k, k_ld, (const float*)v, v_ld,
                                                      qn_w, kn_w, eps, positions, inv_freq, nrot, slots, (float*)q_out,
                                                      (float*)k_cache, (float*)v_cache, Hq, Gk, Gv, D, Dp, Dv, Dvp,
                                                      block_size);
   else
-    qk_norm_rope_kv_kernel<bf16><<<T, 256, sm, s>>>((const bf16*)q, q_ld, (const bf16*)k, k_ld, (const bf16*)v, v_ld,
+    qk_norm_rope_kv_kernel<bf16><<<grid, 256, sm, s>>>((const bf16*)q, q_ld, (const bf16*)k, k_ld, (const bf16*)v, v_ld,
                                                     qn_w, kn_w, eps, positions, inv_freq, nrot, slots, (bf16*)q_out,
                                                     (bf16*)k_cache, (bf16*)v_cache, Hq, Gk, Gv, D, Dp, Dv, Dvp,
                                                     block_size);
@@ -309,14 +447,15 @@ void launch_diff_combine(const float* a, float lam, float eps, float out_mul, co
 }
 
 void launch_glu_clamp(const void* gu, long gu_ld, float limit, float alpha, float up_offset, void* out, int T, int F,
-                      bool f32, hipStream_t s) {
+                      int group, bool f32, hipStream_t s) {
   const long n = (long)T * F;
   if (n <= 0) return;
   const unsigned grid = (unsigned)std::min<long>((n + 255) / 256, 65536);
   if (f32)
-    glu_clamp_kernel<float><<<grid, 256, 0, s>>>((const float*)gu, gu_ld, limit, alpha, up_offset, (float*)out, n, F);
+    glu_clamp_kernel<float><<<grid, 256, 0, s>>>((const float*)gu, gu_ld, limit, alpha, up_offset, (float*)out, n, F,
+                                                 group);
   else
-    glu_clamp_kernel<bf16><<<grid, 256, 0, s>>>((const bf16*)gu, gu_ld, limit, alpha, up_offset, (bf16*)out, n, F);
+    glu_clamp_kernel<bf16><<<grid, 256, 0, s>>>((const bf16*)gu, gu_ld, limit, alpha, up_offset, (bf16*)out, n, F, group);
 }
 
 }  // namespace bfly

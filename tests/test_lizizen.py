@@ -142,7 +142,8 @@ def test_layer_step_norms_token_shift_and_state(target, W):
     assert close(out, O.offset_norm(x[0] + ya[0], wb, eps)[idx.cpu()], dt)
 
 
-@pytest.mark.parametrize("M,F,K,limit", [(5, 7, 13, 1.0), (70, 130, 50, 0.5), (3, 128, 128, 7.0), (300, 192, 64, 1.0)])
+@pytest.mark.parametrize("M,F,K,limit", [(5, 7, 13, 1.0), (70, 130, 50, 0.5), (3, 128, 128, 7.0), (300, 192, 64, 1.0),
+                                         (16, 256, 256, 1.0), (700, 512, 128, 0.75), (40, 1024, 1024, 1.0)])
 def test_clamped_glu_feed_forward(target, M, F, K, limit):
     """min(gate, L) sigmoid(1.702 .) (clamp(up, +-L) + 1) between two biased projections, on shapes
     the tuned matrix-core GEMMs take and on odd ones; inputs large enough that every clamp acts."""
@@ -160,6 +161,20 @@ def test_clamped_glu_feed_forward(target, M, F, K, limit):
     a = ops.glu_clamp(gu[:, :2 * F], limit, 1.702, 1.0)
     y = ops.linear_act(a, g(w["down"]), bias=g(w["down.b"]))
     assert close(y, want, dt, f32_tol=3e-5, bf16_tol=3e-2)
+    # the same through linear_glu, and with gate / up rows in alternating 16-row blocks (the layout
+    # of the GEMMs' fused epilogue, which bf16 shapes the tuned GEMMs take run as one kernel)
+    a2 = ops.linear_glu(g(h), g(wgu), g(bgu), F, limit, 1.702, 1.0, 0)
+    assert close(ops.linear_act(a2, g(w["down"]), bias=g(w["down.b"])), want, dt, f32_tol=3e-5, bf16_tol=3e-2)
+    if F % 16 == 0:
+        wi = ops.interleave_gate_up(w["gate"], w["up"], 16)
+        bi = ops.interleave_gate_up(w["gate.b"][:, None], w["up.b"][:, None], 16)[:, 0]
+        blk = ops.glu_bias_block(g(bi), limit, 1.702, 1.0)
+        if dt == torch.float32:
+            blk = blk.float()          # (an f32 run never takes the fused kernel: plain biases)
+            blk[2 * F:] = 0
+        a3 = ops.linear_glu(g(h), g(wi), blk, F, limit, 1.702, 1.0, 16)
+        assert a3.shape == (M, F)
+        assert close(ops.linear_act(a3, g(w["down"]), bias=g(w["down.b"])), want, dt, f32_tol=3e-5, bf16_tol=3e-2)
 
 
 class Paged:
@@ -473,6 +488,14 @@ def test_padded_head_sizes_round_trip_on_the_gpu(tmp_path):
     W = O.random_weights(cfg, seed=5)
     eng = make_engine(tmp_path, cfg, W, torch.device("cuda"), torch.bfloat16)
     assert eng.model.cache_dims[0] == (32, 32) and eng.model.p["l0.o"].shape == (40, 6 * 32)
+    for lp in eng.model.logical_params():
+        assert torch.equal(lp.get().reshape(W[lp.name].shape).float().cpu(), W[lp.name].float()), lp.name
+    # a width and feed-forward sizes the tuned GEMMs take: gate / up rows in alternating 16-row blocks
+    cfg = cfg_c()
+    W = O.random_weights(cfg, seed=6)
+    eng = make_engine(tmp_path, cfg, W, torch.device("cuda"), torch.bfloat16)
+    assert eng.model.glu_group == {0: 16, 1: 16, 2: 16}
+    assert torch.equal(eng.model.p["l1.gate_up"][16:32].float().cpu(), W["l1.mlp.up"][:16].float())
     for lp in eng.model.logical_params():
         assert torch.equal(lp.get().reshape(W[lp.name].shape).float().cpu(), W[lp.name].float()), lp.name
 
