@@ -309,6 +309,7 @@ class LizizenLM(PackedStack):
         fb.logits_idx names (None: all)."""
         p, c, eps = self.p, self.cfg, self.cfg.norm_eps
         meta = self._step_meta(fb)
+        meta["rope"] = {}
         T, W = fb.num_tokens, c.hidden_size
         if self.has_state and T and not self.state:
             raise RuntimeError("Lizizen: the token-shift pool is not allocated (KVCache state slots)")
@@ -364,8 +365,12 @@ class LizizenLM(PackedStack):
         o2 = o1 + M * G * D
         o3 = o2 + G * Dv
         q, k, v = z[:, :o1].view(T, M * H, D), z[:, o1:o2].view(T, M * G, D), z[:, o2:o3].view(T, G, Dv)
+        # one rotation table per step for all layer runs that share (base, dims)
+        key = (sp["rot_base"], sp["rot_dims"])
+        if key not in meta["rope"]:
+            meta["rope"][key] = ops.rope_table(fb.positions, p[pre + "inv_freq"])
         qp = ops.qk_norm_rope_kv(q, k, v, p[pre + "q.norm"], p[pre + "k.norm"], eps, fb.positions, p[pre + "inv_freq"],
-                                 fb.slots, kc, vc)
+                                 fb.slots, kc, vc, cs=meta["rope"][key])
         a = ops.attn_window_paged(qp, kc, vc, meta["tables"], meta["row_cu"], fb.positions, sp["scale"], NO_WINDOW, 0,
                                   None, row_map=meta["row_map"], chunk=sp["chunk"] if sp["chunk"] < NO_WINDOW else 0,
                                   softcap=sp["softcap"], maps=M, out_dtype=torch.float32)

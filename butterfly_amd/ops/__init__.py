@@ -1100,19 +1100,38 @@ def par_final(x, ya, yb, norm_w, eps: float, offset: float, idx, out_dtype):
     return out
 
 
-def qk_norm_rope_kv(q, k, v, qn_w, kn_w, eps: float, positions, inv_freq, slots, k_cache, v_cache, q_out=None):
+def rope_table(positions, inv_freq):
+    """cs [T, 2, n] f32: cosines and sines of positions[t] * inv_freq[i] (the f32 frequencies; product
+    and evaluation in f64). One table serves every layer of a step that rotates by these
+    frequencies (qk_norm_rope_kv's `cs`). None when nothing rotates."""
+    if inv_freq.numel() == 0:
+        return None
+    if not _gpu(positions):
+        a = positions.double()[:, None] * inv_freq.double()[None]
+        return torch.stack([torch.cos(a), torch.sin(a)], 1).float()
+    cs = _empty(positions.numel(), 2, inv_freq.numel(), dtype=torch.float32, device=positions.device)
+    torch.ops.bfly.rope_table(positions, inv_freq, cs)
+    return cs
+
+
+def qk_norm_rope_kv(q, k, v, qn_w, kn_w, eps: float, positions, inv_freq, slots, k_cache, v_cache, q_out=None, cs=None):
     """Queries and keys prepared per head and the paged append, in one kernel: RMS norm over the
     head with weight qn_w / kn_w [D] f32 (None: no norm), then rotation of the first 2 n dims
     (n = len(inv_freq), may be 0) with dimension i paired with i + n by positions[t] * inv_freq[i].
     q [T, Hq, D] -> q_out [T, Hq, Dp] (Dp = the key cache's row size, zero padded); k [T, Gk, D],
     v [T, Gv, Dv] -> K [blocks, Gk, BS, Dp], V [blocks, Gv, Dvp, BS] at slots[t] >= 0 (the caches'
-    padding keeps the zeros it was allocated with). Returns q_out."""
-    if q_out is None:
+    padding keeps the zeros it was allocated with). `cs`: rope_table(positions, inv_freq), when the
+    caller already has it. Returns q_out, or q itself when the queries need nothing (no norm, no
+    rotation, no padding: only the keys and values are appended)."""
+    plain = qn_w is None and inv_freq.numel() == 0 and k_cache.shape[3] == q.shape[2] and q_out is None
+    if q_out is None and not (plain and _gpu(q)):
         q_out = _empty(q.shape[0], q.shape[1], k_cache.shape[3], dtype=q.dtype, device=q.device)
     if not _gpu(q):
         return ref.qk_norm_rope_kv(q, k, v, qn_w, kn_w, eps, positions, inv_freq, slots, k_cache, v_cache, q_out)
-    torch.ops.bfly.qk_norm_rope_kv(q, k, v, qn_w, kn_w, float(eps), positions, inv_freq, slots, k_cache, v_cache, q_out)
-    return q_out
+    if cs is None:
+        cs = rope_table(positions, inv_freq)
+    torch.ops.bfly.qk_norm_rope_kv(q, k, v, qn_w, kn_w, float(eps), cs, slots, k_cache, v_cache, q_out)
+    return q if q_out is None else q_out
 
 
 def diff_combine(a, lam: float, eps: float, out_mul: float, gate, Dv: int, out_dtype):

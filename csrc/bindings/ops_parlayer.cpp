@@ -101,28 +101,50 @@ void par_final(const Tensor& x, const optional<Tensor>& ya, const optional<Tenso
                          out.data_ptr(), (int)R, (int)W, is_f32(out), cur_stream());
 }
 
+void rope_table(const Tensor& positions, const Tensor& inv_freq, Tensor& cs) {
+  CHK_GPU(positions); CHK_I32(positions); CHK_F32(inv_freq); CHK_F32(cs);
+  const int64_t T = positions.numel(), n = inv_freq.numel();
+  TORCH_CHECK(cs.dim() == 3 && cs.size(0) == T && cs.size(1) == 2 && cs.size(2) == n, "rope_table: cs [T, 2, n]");
+  bfly::launch_rope_table(positions.data_ptr<int>(), inv_freq.data_ptr<float>(), (int)n, cs.data_ptr<float>(), (int)T,
+                          cur_stream());
+}
+
 void qk_norm_rope_kv(const Tensor& q, const Tensor& k, const Tensor& v, const optional<Tensor>& qn_w,
-                     const optional<Tensor>& kn_w, double eps, const Tensor& positions, const Tensor& inv_freq,
-                     const Tensor& slots, Tensor& k_cache, Tensor& v_cache, Tensor& q_out) {
+                     const optional<Tensor>& kn_w, double eps, const optional<Tensor>& cs,
+                     const Tensor& slots, Tensor& k_cache, Tensor& v_cache, const optional<Tensor>& q_out) {
   CHK_GPU(q); CHK_HEADS(q); CHK_HEADS(k); CHK_HEADS(v); CHK_SAME(k, q); CHK_SAME(v, q); CHK_SAME(k_cache, q);
-  CHK_SAME(v_cache, q); CHK_SAME(q_out, q); CHK_I32(positions); CHK_I32(slots); CHK_F32(inv_freq);
+  CHK_SAME(v_cache, q); CHK_I32(slots);
   const int64_t T = q.size(0), Hq = q.size(1), D = q.size(2), Gk = k.size(1), Gv = v.size(1), Dv = v.size(2);
-  TORCH_CHECK(k.size(0) == T && v.size(0) == T && k.size(2) == D && positions.numel() == T && slots.numel() == T,
+  TORCH_CHECK(k.size(0) == T && v.size(0) == T && k.size(2) == D && slots.numel() == T,
               "qk_norm_rope_kv: row counts / head sizes");
-  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.is_contiguous() && v_cache.is_contiguous() &&
-                  q_out.dim() == 3 && q_out.is_contiguous(), "qk_norm_rope_kv: caches / q_out layouts");
+  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.is_contiguous() && v_cache.is_contiguous(),
+              "qk_norm_rope_kv: cache layouts");
   const int64_t bs = k_cache.size(2), Dp = k_cache.size(3), Dvp = v_cache.size(2);
   TORCH_CHECK(k_cache.size(1) == Gk && v_cache.size(1) == Gv && v_cache.size(3) == bs && Dp >= D && Dvp >= Dv &&
                   v_cache.size(0) == k_cache.size(0), "qk_norm_rope_kv: cache shapes K [blocks, Gk, BS, >= D], V [blocks, Gv, >= Dv, BS]");
-  TORCH_CHECK(q_out.size(0) == T && q_out.size(1) == Hq && q_out.size(2) == Dp, "qk_norm_rope_kv: q_out [T, Hq, padded D]");
-  const int64_t nrot = inv_freq.numel();
+  int64_t nrot = 0;
+  const float* csp = nullptr;
+  if (cs.has_value()) {
+    CHK_F32(*cs);
+    TORCH_CHECK(cs->dim() == 3 && cs->size(0) == T && cs->size(1) == 2, "qk_norm_rope_kv: cs [T, 2, n]");
+    nrot = cs->size(2);
+    csp = cs->data_ptr<float>();
+  }
+  void* qo = nullptr;
+  if (q_out.has_value()) {
+    CHK_SAME(*q_out, q);
+    TORCH_CHECK(q_out->dim() == 3 && q_out->is_contiguous() && q_out->size(0) == T && q_out->size(1) == Hq &&
+                    q_out->size(2) == Dp, "qk_norm_rope_kv: q_out [T, Hq, padded D]");
+    qo = q_out->data_ptr();
+  } else {
+    TORCH_CHECK(!qn_w.has_value() && nrot == 0 && Dp == D, "qk_norm_rope_kv: queries that are normed, rotated or padded need q_out");
+  }
   TORCH_CHECK(D >= 1 && Dp <= 512 && 2 * nrot <= D, "qk_norm_rope_kv: head size <= 512, rotated dims <= D");
   const float *qn = nullptr, *kn = nullptr;
   if (qn_w.has_value()) { CHK_F32(*qn_w); TORCH_CHECK(qn_w->numel() == D, "qk_norm_rope_kv: qn_w [D]"); qn = qn_w->data_ptr<float>(); }
   if (kn_w.has_value()) { CHK_F32(*kn_w); TORCH_CHECK(kn_w->numel() == D, "qk_norm_rope_kv: kn_w [D]"); kn = kn_w->data_ptr<float>(); }
   bfly::launch_qk_norm_rope_kv(q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), qn, kn,
-                               (float)eps, positions.data_ptr<int>(), inv_freq.data_ptr<float>(), (int)nrot,
-                               slots.data_ptr<int>(), q_out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), (int)T,
+                               (float)eps, csp, (int)nrot, slots.data_ptr<int>(), qo, k_cache.data_ptr(), v_cache.data_ptr(), (int)T,
                                (int)Hq, (int)Gk, (int)Gv, (int)D, (int)Dp, (int)Dv, (int)Dvp, (int)bs, is_f32(q),
                                cur_stream());
 }
@@ -163,8 +185,8 @@ TORCH_LIBRARY_FRAGMENT(bfly, m) {
         "Tensor positions, Tensor(c!) ha, Tensor(d!)? hb) -> ()");
   m.def("par_final(Tensor x, Tensor? ya, Tensor? yb, Tensor norm_w, float eps, float offset, Tensor? idx, "
         "Tensor(a!) out) -> ()");
-  m.def("qk_norm_rope_kv(Tensor q, Tensor k, Tensor v, Tensor? qn_w, Tensor? kn_w, float eps, Tensor positions, "
-        "Tensor inv_freq, Tensor slots, Tensor(a!) k_cache, Tensor(b!) v_cache, Tensor(c!) q_out) -> ()");
+  m.def("rope_table(Tensor positions, Tensor inv_freq, Tensor(a!) cs) -> ()");
+  m.def("qk_norm_rope_kv(Tensor q, Tensor k, Tensor v, Tensor? qn_w, Tensor? kn_w, float eps, Tensor? cs, Tensor slots, Tensor(a!) k_cache, Tensor(b!) v_cache, Tensor(c!)? q_out) -> ()");
   m.def("diff_combine(Tensor a, float lam, float eps, float out_mul, Tensor? gate, int Dv, Tensor(a!) out) -> ()");
   m.def("glu_clamp(Tensor gu, float limit, float alpha, float up_offset, int group, Tensor(a!) out) -> ()");
 }
@@ -172,6 +194,7 @@ TORCH_LIBRARY_FRAGMENT(bfly, m) {
 TORCH_LIBRARY_IMPL(bfly, CUDA, m) {
   m.impl("par_norm_shift", &par_norm_shift);
   m.impl("par_final", &par_final);
+  m.impl("rope_table", &rope_table);
   m.impl("qk_norm_rope_kv", &qk_norm_rope_kv);
   m.impl("diff_combine", &diff_combine);
   m.impl("glu_clamp", &glu_clamp);

@@ -22,13 +22,16 @@ void launch_par_norm_shift(const float* x, const void* ya, const void* yb, float
 // out[i] = rms(x[r] + (ya[r] + yb[r])) (w + offset), r = idx[i] (idx == nullptr: every row)
 void launch_par_final(const float* x, const void* ya, const void* yb, const float* norm_w, float eps, float offset,
                       const long* idx, void* out, int R, int W, bool f32, hipStream_t s);
+// cs [T, 2, nrot] f32 = cos | sin of positions[t] * inv_freq[f] (f64 product and evaluation)
+void launch_rope_table(const int* positions, const float* inv_freq, int nrot, float* cs, int T, hipStream_t s);
 // Per head: RMS norm over D with weight qn_w / kn_w (nullable: none), then the first 2 nrot dims
-// rotate with dimension i paired with i + nrot by positions[t] * inv_freq[i]. q [T, Hq, D] ->
+// rotate with dimension i paired with i + nrot by the angles of cs (launch_rope_table). q [T, Hq, D] ->
 // q_out [T, Hq, Dp] (zero padded); k [T, Gk, D], v [T, Gv, Dv] -> K [blocks, Gk, BS, Dp],
-// V [blocks, Gv, Dvp, BS] at slots[t] >= 0 (cache padding is left as it is). D <= 512.
+// V [blocks, Gv, Dvp, BS] at slots[t] >= 0 (cache padding is left as it is). D <= 512. q_out == nullptr
+// (allowed without query norm and rotation when Dp == D): the queries stay where they are.
 void launch_qk_norm_rope_kv(const void* q, long q_ld, const void* k, long k_ld, const void* v, long v_ld,
-                            const float* qn_w, const float* kn_w, float eps, const int* positions,
-                            const float* inv_freq, int nrot, const int* slots, void* q_out, void* k_cache,
+                            const float* qn_w, const float* kn_w, float eps, const float* cs, int nrot,
+                            const int* slots, void* q_out, void* k_cache,
                             void* v_cache, int T, int Hq, int Gk, int Gv, int D, int Dp, int Dv, int Dvp, int block_size,
                             bool f32, hipStream_t s);
 // a [T, 2 H, Dvp] f32, heads ordered (head, map): o = a[2h] - lam a[2h + 1] over the first Dv values,

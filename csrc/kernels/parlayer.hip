@@ -228,6 +228,21 @@ __global__ __launch_bounds__(256) void par_final_kernel(const float* __restrict_
 
 constexpr int kMaxHeadLane = 8;      // head sizes up to 512
 
+// cs[t][0][f] = cos(positions[t] * inv_freq[f]), cs[t][1][f] = sin(...): the f32 frequencies, the
+// product and the evaluation in f64. Once per step and rotation (every layer that shares the
+// frequencies reads the same table).
+__global__ void rope_table_kernel(const int* __restrict__ positions, const float* __restrict__ inv_freq, int nrot,
+                                  float* __restrict__ cs, long n) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const long t = i / nrot;
+  const int f = (int)(i % nrot);
+  double sd, cd;
+  sincos((double)positions[t] * (double)inv_freq[f], &sd, &cd);
+  cs[(t * 2) * nrot + f] = (float)cd;
+  cs[(t * 2 + 1) * nrot + f] = (float)sd;
+}
+
 // One workgroup per (token, group of four heads), one wave per head: the query heads, then the key
 // heads; the workgroups of a token share the copy of its value rows. A head is normed in registers
 // (lane l owns dims l, l + 64, ...), staged in LDS so that a rotated dimension finds its partner,
@@ -237,29 +252,20 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_kernel(const T* __restric
                                                               long k_ld, const T* __restrict__ v, long v_ld,
                                                               const float* __restrict__ qn_w,
                                                               const float* __restrict__ kn_w, float eps,
-                                                              const int* __restrict__ positions,
-                                                              const float* __restrict__ inv_freq, int nrot,
+                                                              const float* __restrict__ cs, int nrot,
                                                               const int* __restrict__ slots, T* __restrict__ q_out,
                                                               T* __restrict__ k_cache, T* __restrict__ v_cache, int Hq,
                                                               int Gk, int Gv, int D, int Dp, int Dv, int Dvp, int bs) {
-  extern __shared__ float smem[];        // head staging [4][D] | cos [nrot] | sin [nrot]
+  extern __shared__ float smem[];        // head staging [4][D]
   const long t = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   float* sh = smem + (long)wave * D;
-  float* scos = smem + 4L * D;
-  float* ssin = scos + nrot;
-  const int p = positions[t];
-  // the token's angles once for all heads: f64 product and evaluation of the f32 frequencies
-  for (int f = threadIdx.x; f < nrot; f += blockDim.x) {
-    double sd, cd;
-    sincos((double)p * (double)inv_freq[f], &sd, &cd);
-    scos[f] = (float)cd;
-    ssin[f] = (float)sd;
-  }
-  __syncthreads();
+  const float* scos = cs + t * 2 * nrot;       // the token's row of the step's rotation table
+  const float* ssin = scos + nrot;
   const int slot = slots ? slots[t] : -1;
   const long blk = slot >= 0 ? slot / bs : 0, off = slot >= 0 ? slot % bs : 0;
-  const int hh = 4 * blockIdx.y + wave;
+  // q_out == nullptr: the queries need nothing (no norm, no rotation, no padding); key heads only
+  const int hh = 4 * blockIdx.y + wave + (q_out ? 0 : Hq);
   if (hh < Hq + Gk && (hh < Hq || slot >= 0)) {
     const bool isq = hh < Hq;
     const int h = isq ? hh : hh - Hq;
@@ -415,23 +421,29 @@ void launch_par_final(const float* x, const void* ya, const void* yb, const floa
 }
 
 void launch_qk_norm_rope_kv(const void* q, long q_ld, const void* k, long k_ld, const void* v, long v_ld,
-                            const float* qn_w, const float* kn_w, float eps, const int* positions,
-                            const float* inv_freq, int nrot, const int* slots, void* q_out, void* k_cache,
+                            const float* qn_w, const float* kn_w, float eps, const float* cs, int nrot,
+                            const int* slots, void* q_out, void* k_cache,
                             void* v_cache, int T, int Hq, int Gk, int Gv, int D, int Dp, int Dv, int Dvp, int block_size,
                             bool f32, hipStream_t s) {
   if (T <= 0) return;
-  const size_t sm = (size_t)(4 * D + 2 * nrot) * sizeof(float);
-  const dim3 grid(T, (Hq + Gk + 3) / 4);
+  const size_t sm = (size_t)(4 * D) * sizeof(float);
+  const dim3 grid(T, ((q_out ? Hq : 0) + Gk + 3) / 4);
   if (f32)
     qk_norm_rope_kv_kernel<float><<<grid, 256, sm, s>>>((const float*)q, q_ld, (const float*)k, k_ld, (const float*)v, v_ld,
-                                                     qn_w, kn_w, eps, positions, inv_freq, nrot, slots, (float*)q_out,
+                                                     qn_w, kn_w, eps, cs, nrot, slots, (float*)q_out,
                                                      (float*)k_cache, (float*)v_cache, Hq, Gk, Gv, D, Dp, Dv, Dvp,
                                                      block_size);
   else
     qk_norm_rope_kv_kernel<bf16><<<grid, 256, sm, s>>>((const bf16*)q, q_ld, (const bf16*)k, k_ld, (const bf16*)v, v_ld,
-                                                    qn_w, kn_w, eps, positions, inv_freq, nrot, slots, (bf16*)q_out,
+                                                    qn_w, kn_w, eps, cs, nrot, slots, (bf16*)q_out,
                                                     (bf16*)k_cache, (bf16*)v_cache, Hq, Gk, Gv, D, Dp, Dv, Dvp,
                                                     block_size);
+}
+
+void launch_rope_table(const int* positions, const float* inv_freq, int nrot, float* cs, int T, hipStream_t s) {
+  const long n = (long)T * nrot;
+  if (n <= 0) return;
+  rope_table_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(positions, inv_freq, nrot, cs, n);
 }
 
 void launch_diff_combine(const float* a, float lam, float eps, float out_mul, const void* gate, long gate_ld,
