@@ -243,11 +243,13 @@ __global__ void rope_table_kernel(const int* __restrict__ positions, const float
   cs[(t * 2 + 1) * nrot + f] = (float)sd;
 }
 
-// One workgroup per (token, group of four heads), one wave per head: the query heads, then the key
+// One workgroup per (token, group of 4 HPW heads), HPW heads per wave: the query heads, then the key
 // heads; the workgroups of a token share the copy of its value rows. A head is normed in registers
-// (lane l owns dims l, l + 64, ...), staged in LDS so that a rotated dimension finds its partner,
-// and leaves rotated.
-template <typename T>
+// (lane l owns dims l, l + 64, ...: NL per lane), staged in LDS so that a rotated dimension finds its
+// partner, and leaves rotated. A wave's HPW heads go through each phase together (all loads, all
+// reductions, all hand-overs, all stores), so their latencies overlap: large steps take HPW = 4,
+// steps of few rows HPW = 1 (more workgroups).
+template <typename T, int HPW, int NL>
 __global__ __launch_bounds__(256) void qk_norm_rope_kv_kernel(const T* __restrict__ q, long q_ld, const T* __restrict__ k,
                                                               long k_ld, const T* __restrict__ v, long v_ld,
                                                               const float* __restrict__ qn_w,
@@ -256,70 +258,88 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_kernel(const T* __restric
                                                               const int* __restrict__ slots, T* __restrict__ q_out,
                                                               T* __restrict__ k_cache, T* __restrict__ v_cache, int Hq,
                                                               int Gk, int Gv, int D, int Dp, int Dv, int Dvp, int bs) {
-  extern __shared__ float smem[];        // head staging [4][D]
+  extern __shared__ float smem[];        // head staging [4][HPW][D]
   const long t = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  float* sh = smem + (long)wave * D;
   const float* scos = cs + t * 2 * nrot;       // the token's row of the step's rotation table
   const float* ssin = scos + nrot;
   const int slot = slots ? slots[t] : -1;
   const long blk = slot >= 0 ? slot / bs : 0, off = slot >= 0 ? slot % bs : 0;
   // q_out == nullptr: the queries need nothing (no norm, no rotation, no padding); key heads only
-  const int hh = 4 * blockIdx.y + wave + (q_out ? 0 : Hq);
-  if (hh < Hq + Gk && (hh < Hq || slot >= 0)) {
-    const bool isq = hh < Hq;
-    const int h = isq ? hh : hh - Hq;
-    const T* src = isq ? q + t * q_ld + (long)h * D : k + t * k_ld + (long)h * D;
-    const float* nw = isq ? qn_w : kn_w;
-    float val[kMaxHeadLane];
+  const int h0 = 4 * HPW * blockIdx.y + wave + (q_out ? 0 : Hq);
+  float val[HPW][NL];
+  bool on[HPW];
+#pragma unroll
+  for (int u = 0; u < HPW; ++u) {
+    const int hh = h0 + 4 * u;
+    on[u] = hh < Hq + Gk && (hh < Hq || slot >= 0);
+    const T* src = hh < Hq ? q + t * q_ld + (long)hh * D : k + t * k_ld + (long)(hh - Hq) * D;
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const int d = lane + 64 * i;
+      val[u][i] = (on[u] && d < D) ? (float)src[d] : 0.f;
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < HPW; ++u) {
+    const float* nw = h0 + 4 * u < Hq ? qn_w : kn_w;
+    if (!nw || !on[u]) continue;
     float ss = 0.f;
 #pragma unroll
-    for (int i = 0; i < kMaxHeadLane; ++i) {
+    for (int i = 0; i < NL; ++i) ss = fmaf(val[u][i], val[u][i], ss);
+    const float r = 1.f / sqrtf(wave_sum(ss) / (float)D + eps);
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
       const int d = lane + 64 * i;
-      val[i] = d < D ? (float)src[d] : 0.f;
-      ss = fmaf(val[i], val[i], ss);
+      if (d < D) val[u][i] = val[u][i] * r * nw[d];
     }
-    if (nw) {
-      const float r = 1.f / sqrtf(wave_sum(ss) / (float)D + eps);
+  }
+  if (nrot > 0) {
 #pragma unroll
-      for (int i = 0; i < kMaxHeadLane; ++i) {
+    for (int u = 0; u < HPW; ++u) {
+      float* sh = smem + (long)(wave * HPW + u) * D;
+#pragma unroll
+      for (int i = 0; i < NL; ++i) {
         const int d = lane + 64 * i;
-        if (d < D) val[i] = val[i] * r * nw[d];
+        if (d < D) sh[d] = val[u][i];
       }
     }
-    if (nrot > 0) {
+    __builtin_amdgcn_wave_barrier();
+    __threadfence_block();
 #pragma unroll
-      for (int i = 0; i < kMaxHeadLane; ++i) {
-        const int d = lane + 64 * i;
-        if (d < D) sh[d] = val[i];
-      }
-      __builtin_amdgcn_wave_barrier();
-      __threadfence_block();
+    for (int i = 0; i < NL; ++i) {
+      const int d = lane + 64 * i;
+      if (d < 2 * nrot) {
+        const int f = d < nrot ? d : d - nrot;
+        const float c = scos[f], sn = ssin[f];
 #pragma unroll
-      for (int i = 0; i < kMaxHeadLane; ++i) {
-        const int d = lane + 64 * i;
-        if (d < 2 * nrot) {
-          const int f = d < nrot ? d : d - nrot;
-          const float c = scos[f], sn = ssin[f];
-          // pair (u, w) = dims (f, f + nrot): u' = u c - w s, w' = w c + u s
-          val[i] = d < nrot ? val[i] * c - sh[d + nrot] * sn : val[i] * c + sh[d - nrot] * sn;
+        for (int u = 0; u < HPW; ++u) {
+          const float* sh = smem + (long)(wave * HPW + u) * D;
+          // pair (a, b) = dims (f, f + nrot): a' = a c - b s, b' = b c + a s
+          val[u][i] = d < nrot ? val[u][i] * c - sh[d + nrot] * sn : val[u][i] * c + sh[d - nrot] * sn;
         }
       }
-      __builtin_amdgcn_wave_barrier();
     }
-    if (isq) {
-      T* dst = q_out + (t * Hq + h) * Dp;
+  }
 #pragma unroll
-      for (int i = 0; i < kMaxHeadLane; ++i) {
-        const int d = lane + 64 * i;
-        if (d < Dp) dst[d] = (T)(d < D ? val[i] : 0.f);
+  for (int u = 0; u < HPW; ++u) {
+    if (!on[u]) continue;
+    const int hh = h0 + 4 * u;
+    if (hh < Hq) {
+      T* dst = q_out + (t * Hq + hh) * Dp;
+      for (int d = lane; d < Dp; d += 64) {       // (the padding past 64 NL stays in this loop's zero branch)
+        float x = 0.f;
+#pragma unroll
+        for (int i = 0; i < NL; ++i)
+          if (d == lane + 64 * i) x = val[u][i];
+        dst[d] = (T)(d < D ? x : 0.f);
       }
     } else {
-      T* dst = k_cache + ((blk * Gk + h) * bs + off) * Dp;
+      T* dst = k_cache + ((blk * Gk + (hh - Hq)) * bs + off) * Dp;
 #pragma unroll
-      for (int i = 0; i < kMaxHeadLane; ++i) {
+      for (int i = 0; i < NL; ++i) {
         const int d = lane + 64 * i;
-        if (d < D) dst[d] = (T)val[i];
+        if (d < D) dst[d] = (T)val[u][i];
       }
     }
   }
@@ -420,24 +440,40 @@ void launch_par_final(const float* x, const void* ya, const void* yb, const floa
                                              W);
 }
 
+template <typename T>
+static void qk_launch(const T* q, long q_ld, const T* k, long k_ld, const T* v, long v_ld, const float* qn_w,
+                      const float* kn_w, float eps, const float* cs, int nrot, const int* slots, T* q_out, T* k_cache,
+                      T* v_cache, int Tn, int Hq, int Gk, int Gv, int D, int Dp, int Dv, int Dvp, int bs, hipStream_t s) {
+  const int heads = (q_out ? Hq : 0) + Gk;
+  const bool big = (long)Tn * heads >= 4096;       // enough waves either way: several heads per wave
+  const int hpw = big ? 4 : 1;
+  const dim3 grid(Tn, (heads + 4 * hpw - 1) / (4 * hpw));
+  const size_t sm = (size_t)(4 * hpw * D) * sizeof(float);
+#define BFLY_QK(HPW, NL)                                                                                          \
+  qk_norm_rope_kv_kernel<T, HPW, NL><<<grid, 256, sm, s>>>(q, q_ld, k, k_ld, v, v_ld, qn_w, kn_w, eps, cs, nrot, slots, \
+                                                          q_out, k_cache, v_cache, Hq, Gk, Gv, D, Dp, Dv, Dvp, bs)
+#define BFLY_QKN(HPW)              \
+  if (D <= 64) BFLY_QK(HPW, 1);    \
+  else if (D <= 128) BFLY_QK(HPW, 2); \
+  else if (D <= 256) BFLY_QK(HPW, 4); \
+  else BFLY_QK(HPW, 8)
+  if (big) { BFLY_QKN(4); } else { BFLY_QKN(1); }
+#undef BFLY_QKN
+#undef BFLY_QK
+}
+
 void launch_qk_norm_rope_kv(const void* q, long q_ld, const void* k, long k_ld, const void* v, long v_ld,
                             const float* qn_w, const float* kn_w, float eps, const float* cs, int nrot,
                             const int* slots, void* q_out, void* k_cache,
                             void* v_cache, int T, int Hq, int Gk, int Gv, int D, int Dp, int Dv, int Dvp, int block_size,
                             bool f32, hipStream_t s) {
   if (T <= 0) return;
-  const size_t sm = (size_t)(4 * D) * sizeof(float);
-  const dim3 grid(T, ((q_out ? Hq : 0) + Gk + 3) / 4);
   if (f32)
-    qk_norm_rope_kv_kernel<float><<<grid, 256, sm, s>>>((const float*)q, q_ld, (const float*)k, k_ld, (const float*)v, v_ld,
-                                                     qn_w, kn_w, eps, cs, nrot, slots, (float*)q_out,
-                                                     (float*)k_cache, (float*)v_cache, Hq, Gk, Gv, D, Dp, Dv, Dvp,
-                                                     block_size);
+    qk_launch<float>((const float*)q, q_ld, (const float*)k, k_ld, (const float*)v, v_ld, qn_w, kn_w, eps, cs, nrot, slots,
+                     (float*)q_out, (float*)k_cache, (float*)v_cache, T, Hq, Gk, Gv, D, Dp, Dv, Dvp, block_size, s);
   else
-    qk_norm_rope_kv_kernel<bf16><<<grid, 256, sm, s>>>((const bf16*)q, q_ld, (const bf16*)k, k_ld, (const bf16*)v, v_ld,
-                                                    qn_w, kn_w, eps, cs, nrot, slots, (bf16*)q_out,
-                                                    (bf16*)k_cache, (bf16*)v_cache, Hq, Gk, Gv, D, Dp, Dv, Dvp,
-                                                    block_size);
+    qk_launch<bf16>((const bf16*)q, q_ld, (const bf16*)k, k_ld, (const bf16*)v, v_ld, qn_w, kn_w, eps, cs, nrot, slots,
+                    (bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, T, Hq, Gk, Gv, D, Dp, Dv, Dvp, block_size, s);
 }
 
 void launch_rope_table(const int* positions, const float* inv_freq, int nrot, float* cs, int T, hipStream_t s) {
