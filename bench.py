@@ -208,9 +208,9 @@ def run_mixer_compare(a) -> int:
             # dense clamped-GLU feed-forwards, beside plain GQA attention of the same heads (causal where
             # the biased layers are, a window of the chunk size where the chunked ones are) with dense
             # feed-forwards of the same parameter count (two matrices of 3/2 the width), one stream
-            bia = {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5, "q_temp": {"coef": 0.1, "every": 256}}
-            dif = {"heads": H // 2, "kv_heads": max(G // 2, 1), "dim": D, "vdim": 2 * D, "scale": D ** -0.5, "diff": 0.6,
-                   "mask": {"size": win}, "rot": {"dims": D // 2, "base": 1e6}, "softcap": 50.0}
+            bia = {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5, "q_temp": {"coef": 0.1, "every": 128}}
+            dif = {"heads": H // 2, "kv_heads": max(G // 2, 1), "dim": D, "vdim": 2 * D, "scale": D ** -0.5, "diff": 0.5,
+                   "mask": {"size": win}, "rot": {"dims": D // 2, "base": 1e6}, "softcap": 30.0}
             glu = {"kind": "dense", "ff": dff, "limit": 7.0}
             liz = ModelConfig.from_lizizen({"architecture": "Lizizen", "vocab": 32000, "width": W, "norm": {"eps": 1e-6},
                                             "layers": [{"type": t, "mixer": m, "mlp": glu} for t, m in

@@ -219,7 +219,7 @@ STEPS = [[(0, 150), (1, 1)], [(0, 2), (1, 1), (2, 40)], [(0, 1), (1, 2)], [(0, 1
          [(0, 1), (1, 26)], [(0, 64)]] + [[(0, 1), (2, 1)]] * 8
 
 
-@pytest.mark.parametrize("H,G,D,Dv,coef,every", [(6, 3, 20, 12, 0.5, 7), (8, 2, 64, 64, 0.25, 100), (4, 4, 48, 96, 0.0, 1),
+@pytest.mark.parametrize("H,G,D,Dv,coef,every", [(6, 3, 20, 12, 0.5, 7), (8, 2, 64, 64, 0.25, 100), (4, 4, 40, 96, 0.0, 1),
                                                  (2, 1, 128, 32, 1.0, 1)])
 def test_distance_biased_attention_with_sink(target, H, G, D, Dv, coef, every):
     """Causal attention over hundreds of cached keys in prompts, portions and decoded rows: queries
@@ -260,7 +260,7 @@ def test_distance_biased_attention_with_sink(target, H, G, D, Dv, coef, every):
         assert close(torch.cat(got[s]), want[s], dt, f32_tol=2e-5, bf16_tol=2.5e-2), f"sequence {s}"
 
 
-@pytest.mark.parametrize("H,G,D,Dv,chunk,cap,dims", [(3, 1, 20, 12, 7, 3.0, 8), (4, 2, 64, 64, 40, 0.0, 64), (2, 2, 48, 96, 64, 50.0, 24),
+@pytest.mark.parametrize("H,G,D,Dv,chunk,cap,dims", [(3, 1, 20, 12, 7, 3.0, 8), (4, 2, 64, 64, 40, 0.0, 64), (2, 2, 40, 96, 64, 30.0, 20),
                                                      (4, 2, 32, 128, 33, 2.0, 0), (2, 1, 16, 16, 1, 0.0, 4)])
 def test_chunked_two_map_attention(target, H, G, D, Dv, chunk, cap, dims):
     """Two maps per head over shared values, normed and half-rotated, keys of the query's own chunk
@@ -305,6 +305,60 @@ def test_chunked_two_map_attention(target, H, G, D, Dv, chunk, cap, dims):
             r += c
             at[s] += c
     for s in range(3):
+        assert close(torch.cat(got[s]), want[s], dt, f32_tol=3e-5, bf16_tol=4e-2), f"sequence {s}"
+
+
+@pytest.mark.parametrize("kind", ["biased", "two_map"])
+def test_attention_decoding_over_long_contexts(target, kind):
+    """Decoded rows over a thousand cached tokens (on the GPU the pages of a row are then split over
+    several workgroups and merged), two sequences per step, then a short portion: a far key, the
+    first key, the sink's share and a long chunk's first key are all met."""
+    dev, dt = target
+    lens = [1060, 700]
+    steps = [[(0, 1000), (1, 650)]] + [[(0, 1), (1, 1)]] * 30 + [[(0, 30), (1, 20)]]
+    if kind == "biased":
+        H, G, D, Dv, scale = 4, 2, 64, 64, 0.2
+        q = [rnd(n, H, D, seed=140 + s) for s, n in enumerate(lens)]
+        k = [rnd(n, G, D, seed=150 + s) for s, n in enumerate(lens)]
+        v = [rnd(n, G, Dv, seed=160 + s) for s, n in enumerate(lens)]
+        aim(q[0], k[0], [(1005, 0), (1010, 17), (1020, 999), (1029, 512), (1040, 31)], scale, H // G)
+        aim(q[1], k[1], [(660, 1), (679, 640), (690, 300)], scale, H // G)
+        r1, r2 = bf(0.2 + 0.8 * torch.rand(H, dtype=F64)), bf(0.05 + 0.5 * torch.rand(H, dtype=F64))
+        want = [O.biased_attend(q[s], k[s], v[s], r1, r2, scale, 0.5, 300) for s in range(2)]
+        cache = Paged(lens, G, G, D, Dv, dev, dt, seed=5)
+        prep = (None, None, 1e-5, torch.zeros(0, dtype=torch.float32, device=dev))
+        attn = dict(scale=scale, window=1 << 30, keep_first=0, sink=torch.zeros(H, dtype=torch.float32, device=dev),
+                    dist_bias=(r1.float().to(dev), r2.float().to(dev)), q_temp=(0.5, 300))
+        qs, ks = q, k
+    else:
+        H, G, D, Dv, chunk, cap, dims, base, eps = 2, 1, 32, 64, 600, 8.0, 16, 1e4, 1e-5
+        scale = 14.0 / D
+        q = [rnd(n, H, 2, D, seed=170 + s) for s, n in enumerate(lens)]
+        k = [rnd(n, G, 2, D, seed=180 + s) for s, n in enumerate(lens)]
+        v = [rnd(n, G, Dv, seed=190 + s) for s, n in enumerate(lens)]
+        for s, rows in ((0, range(1000, 1060, 7)), (1, range(650, 700, 5))):
+            for i in rows:
+                j = i - i % chunk if i % 2 else i - i % chunk - 1          # first key of the chunk / the key before it
+                q[s][i] = bf(k[s][j, 0] * 3.0).expand(H, 2, D)
+        qn, kn = bf(1 + 0.2 * torch.randn(D, dtype=F64)), bf(1 + 0.2 * torch.randn(D, dtype=F64))
+        want = [O.chunk_attend(O.normed_rotated(q[s], qn, eps, base, dims), O.normed_rotated(k[s], kn, eps, base, dims),
+                               v[s], scale, cap, chunk).reshape(lens[s], 2 * H, Dv) for s in range(2)]
+        cache = Paged(lens, 2 * G, G, D, Dv, dev, dt, seed=6)
+        inv = torch.tensor([base ** (-2.0 * i / dims) for i in range(dims // 2)], dtype=F64).float().to(dev)
+        prep = (qn.float().to(dev), kn.float().to(dev), eps, inv)
+        attn = dict(scale=scale, window=1 << 30, keep_first=0, sink=None, chunk=chunk, softcap=cap, maps=2,
+                    out_dtype=torch.float32)
+        qs, ks = [x.reshape(x.shape[0], -1, D) for x in q], [x.reshape(x.shape[0], -1, D) for x in k]
+    at, got = [0, 0], [[], []]
+    for step in steps:
+        out = cache.step(step, at, qs, ks, v, prep, attn)
+        r = 0
+        for s, c in step:
+            got[s].append(out[r:r + c, :, :Dv])
+            r += c
+            at[s] += c
+    assert at == lens
+    for s in range(2):
         assert close(torch.cat(got[s]), want[s], dt, f32_tol=3e-5, bf16_tol=4e-2), f"sequence {s}"
 
 
@@ -369,7 +423,7 @@ def cfg_a():
     shorter than a page; a layer without feed-forward; the middle span of layers runs three times."""
     return O.config([
         O.biased_layer(6, 3, 12, 20, 0.3, 0.5, 5, O.dense(56, 1.0)),
-        O.diff_layer(3, 1, 10, 6, 0.4, 0.6, 7, 100.0, 4, 3.0, O.dense(24, 0.5)),
+        O.diff_layer(3, 1, 10, 6, 0.4, 0.65, 7, 100.0, 4, 3.0, O.dense(24, 0.5)),
         O.biased_layer(2, 2, 8, 8, 0.25, 0.25, 16, None),
         O.diff_layer(4, 2, 6, 14, 0.5, 0.2, 40, 1e4, 6, 20.0, O.dense(40, 2.0)),
     ], width=40, vocab=70, eps=1e-5, loop=(1, 3, 3))
@@ -398,8 +452,8 @@ def cfg_c():
     run twice."""
     return O.config([
         O.biased_layer(8, 2, 64, 64, 0.125, 0.5, 48, O.dense(256, 1.0)),
-        O.diff_layer(4, 2, 32, 128, 0.18, 0.6, 40, 5e5, 16, 30.0, O.dense(128, 1.0)),
-        O.diff_layer(2, 1, 128, 32, 0.09, 0.4, 64, 1e4, 128, 50.0, O.dense(256, 3.0)),
+        O.diff_layer(4, 2, 32, 128, 0.18, 0.55, 40, 2e5, 16, 30.0, O.dense(128, 1.0)),
+        O.diff_layer(2, 1, 128, 32, 0.09, 0.4, 64, 1e4, 128, 45.0, O.dense(256, 3.0)),
     ], width=128, vocab=256, eps=1e-5, loop=(0, 2, 2))
 
 
