@@ -16,7 +16,7 @@ from typing import Any, Optional
 @dataclass
 class ModelConfig:
     name: str
-    arch: str                       # "llama" | "gpt2" | "mixtral" | "nesizen" | "zinesun" | "lizizen"
+    arch: str                       # "llama" | "gpt2" | "mixtral" | "nesizen" | "zinesun" | "lizizen" | "gevipel"
     vocab_size: int
     hidden_size: int
     intermediate_size: int
@@ -45,6 +45,9 @@ class ModelConfig:
     # layer indices in the order they run, when a span of layers repeats with the same weights
     # (every run has its own cache and state); None: each layer once, in order
     layer_runs: Optional[list] = None
+    residual_mult: float = 1.0      # a sublayer's (normed) output is multiplied by this before the residual sum
+    loop_start: int = -1            # >= 0: first layer of the repeated span (the embedding output re-enters
+                                    # the residual before every repetition of it but the first)
 
     # ---- derived quantities ------------------------------------------------------------
     @property
@@ -95,13 +98,13 @@ class ModelConfig:
         if self.layer_specs:
             # a latent-attention layer caches its latent twice (key rows and transposed value
             # rows) and the shared rotated key part once
-            return sum(sp["kv_heads"] * (sp["dim"] + sp["vdim"]) * dtype_bytes for sp in self.layer_specs
+            runs = [self.layer_specs[i] for i in (self.layer_runs or range(len(self.layer_specs)))]
+            return sum(sp["kv_heads"] * (sp["dim"] + sp["vdim"]) * dtype_bytes for sp in runs
                        if sp["type"] == "attention" and sp["kv_from"] is None) + \
-                sum((2 * sp["kv_rank"] + sp["rot_dim"]) * dtype_bytes for sp in self.layer_specs
+                sum((2 * sp["kv_rank"] + sp["rot_dim"]) * dtype_bytes for sp in runs
                     if sp["type"] == "latent_attention") + \
-                sum(sp["kv_heads"] * (sp["maps"] * sp["dim"] + sp["vdim"]) * dtype_bytes
-                    for sp in (self.layer_specs[i] for i in (self.layer_runs or range(len(self.layer_specs))))
-                    if sp["type"] in ("biased_attention", "diff_attention"))
+                sum(sp["kv_heads"] * (sp["maps"] * sp["dim"] + sp["vdim"]) * dtype_bytes for sp in runs
+                    if sp["type"] in ("biased_attention", "diff_attention", "sloped_attention"))
         return 2 * self.num_layers * self.kv_size * dtype_bytes
 
     # ---- (de)serialisation -------------------------------------------------------------
@@ -200,6 +203,50 @@ class ModelConfig:
                    layer_specs=specs, layer_runs=runs)
 
     @classmethod
+    def from_gevipel(cls, js: dict, name: str = "gevipel") -> "ModelConfig":
+        """Map a Gevipel config.json ("architecture": "Gevipel") to ModelConfig: layers with a layer
+        norm before and after every sublayer and a constant factor on the normed sublayer output,
+        three mixers (sliding-window attention with a linear distance bias whose values are the keys,
+        "attention"; the gated delta rule with short convolutions, "delta"; causal latent attention
+        with a sink, "latent_attention"), routed squared-ReLU experts chosen with a score correction,
+        a scaled embedding, and a span of layers that may run several times with the same weights
+        ("loop"), the embedding output re-entering before every repetition. Every size and per-layer
+        constant is taken from the file."""
+        kinds = {"attention": "sloped_attention", "delta": "delta", "latent_attention": "latent_attention"}
+        specs = []
+        for i, L in enumerate(js["layers"]):
+            if L["type"] not in kinds:
+                raise ValueError(f"layer {i}: Gevipel has no mixer {L['type']!r}")
+            sp = layer_spec(i, {**L, "type": kinds[L["type"]]})
+            if sp["ffn"]:
+                if sp["ffn"]["kind"] != "moe":
+                    raise ValueError(f"layer {i}: Gevipel has no feed-forward {sp['ffn']['kind']!r}")
+                sp["ffn"]["glu"] = False          # experts are W_down relu(W_up h)^2
+            specs.append(sp)
+        n = len(specs)
+        runs, start = list(range(n)), -1
+        lp = js.get("loop")
+        if lp:
+            a, b, times = int(lp["start"]), int(lp["stop"]), int(lp.get("times", 1))
+            if not (0 <= a <= b <= n) or times < 1:
+                raise ValueError("loop: need 0 <= start <= stop <= layers and times >= 1")
+            runs = list(range(a)) + list(range(a, b)) * times + list(range(b, n))
+            start = a if b > a else -1
+        mx = lambda key: max([sp.get(key) or 0 for sp in specs] + [0])  # noqa: E731
+        moe = [sp["ffn"] for sp in specs if sp["ffn"]]
+        return cls(name=name, arch="gevipel", vocab_size=int(js["vocab"]), hidden_size=int(js["width"]),
+                   intermediate_size=max([m["ff"] for m in moe] + [0]),
+                   num_layers=n, num_heads=mx("heads"), num_kv_heads=max(mx("kv_heads"), 1),
+                   head_dim=max(mx("dim") + mx("rot_dim"), mx("kv_rank") + mx("rot_dim"), mx("vdim")),
+                   max_position=1 << 30, norm_eps=float(js["norm"]["eps"]),
+                   norm="layer", act="relu2", pos_emb="rope", tie_embeddings=False,
+                   num_experts=max([m["experts"] for m in moe] + [0]),
+                   experts_per_token=max([m["top"] for m in moe] + [0]),
+                   layer_specs=specs, layer_runs=runs, loop_start=start,
+                   embed_scale=float((js.get("embedding") or {}).get("scale", 1.0)),
+                   residual_mult=float(js.get("residual_mult", 1.0)))
+
+    @classmethod
     def from_model_dir(cls, path, name: Optional[str] = None) -> "ModelConfig":
         """config.json of a model folder -> ModelConfig; the "architecture" / "model_type" key
         chooses the family."""
@@ -212,6 +259,8 @@ class ModelConfig:
             return cls.from_zinesun(js, name=name)
         if family == "lizizen":
             return cls.from_lizizen(js, name=name)
+        if family == "gevipel":
+            return cls.from_gevipel(js, name=name)
         return cls.from_hf(js, name=name)
 
     @classmethod
@@ -260,7 +309,11 @@ def layer_spec(index: int, L: dict) -> dict:
     qt_every); "diff_attention": two softmax maps per head over the same values, combined as a
     difference (heads, kv_heads, dim, vdim, maps = 2, scale, diff, chunk, rot_dims, rot_base,
     softcap), with normed and half-rotated queries and keys, visible inside chunks of `chunk`
-    positions. `ffn`: None, or kind "dense" (ff) / "glu" (dense clamped GLU with biases: ff,
+    positions; "sloped_attention": sliding-window softmax attention without rotation whose values
+    are the keys as projected, with normed queries and keys, a linear per-head distance bias and the
+    query temperature (heads, kv_heads, dim, vdim = dim, scale, window, qt_coef, qt_every); "delta":
+    the gated delta rule with short convolutions on its query, key and value rows (heads, kv_heads,
+    dim, vdim, taps). `ffn`: None, or kind "dense" (ff) / "glu" (dense clamped GLU with biases: ff,
     limit) / "moe" (ff, limit or None for unclamped experts, experts, top)."""
     m, t = L["mixer"], L["type"]
     sp = {"index": index, "type": t, "heads": int(m["heads"]), "dim": int(m["dim"]), "vdim": int(m["vdim"]),
@@ -291,16 +344,30 @@ def layer_spec(index: int, L: dict) -> dict:
             raise ValueError(f"layer {index}: window must be >= 1 and keep_first >= 0")
         if sp["heads"] % sp["kv_heads"] or sp["rot_dims"] % 2 or sp["rot_dims"] > sp["dim"]:
             raise ValueError(f"layer {index}: bad attention sizes")
+    elif t == "sloped_attention":
+        qt = m.get("q_temp") or {"coef": 0.0, "every": 1}            # absent: no temperature
+        mask = m.get("mask") or {"size": 1 << 30}                    # absent: plain causal attention
+        sp.update(kv_heads=int(m.get("kv_heads", m["heads"])), scale=float(m.get("scale", sp["dim"] ** -0.5)),
+                  window=int(mask["size"]), qt_coef=float(qt.get("coef", 0.0)), qt_every=int(qt.get("every", 1)))
+        if sp["kv_heads"] < 1 or sp["heads"] % sp["kv_heads"] or sp["qt_every"] < 1 or sp["window"] < 1:
+            raise ValueError(f"layer {index}: bad attention sizes")
+        if sp["vdim"] != sp["dim"]:
+            raise ValueError(f"layer {index}: the values are the keys, so vdim must equal dim")
+    elif t == "delta":
+        sp.update(kv_heads=int(m.get("kv_heads", m["heads"])), taps=int(m.get("conv", 1)))
+        if sp["kv_heads"] < 1 or sp["heads"] % sp["kv_heads"] or sp["taps"] < 1:
+            raise ValueError(f"layer {index}: bad delta-rule sizes")
     elif t == "latent_attention":
         rot = m.get("rot") or {}
         mask = m.get("mask") or {"size": 1 << 30}
-        sp.update(rot_dim=int(m.get("rot_dim", 0)), kv_rank=int(m["kv_rank"]), q_rank=int(m["q_rank"]),
+        # q_rank 0: the queries are projected from the mixer's input directly
+        sp.update(rot_dim=int(m.get("rot_dim", 0)), kv_rank=int(m["kv_rank"]), q_rank=int(m.get("q_rank", 0)),
                   rot_base=float(rot.get("base", 10000.0)), rot_dims=int(rot.get("dims", m.get("rot_dim", 0))),
                   scale=float(m.get("scale", (sp["dim"] + int(m.get("rot_dim", 0))) ** -0.5)),
                   window=int(mask["size"]))
         if sp["rot_dims"] > sp["rot_dim"] or sp["rot_dims"] % 2:
             raise ValueError(f"layer {index}: rot.dims must be even and at most rot_dim")
-        if sp["window"] < 1 or min(sp["kv_rank"], sp["q_rank"], sp["dim"] + sp["rot_dim"]) < 1:
+        if sp["window"] < 1 or min(sp["kv_rank"], sp["dim"] + sp["rot_dim"]) < 1 or sp["q_rank"] < 0:
             raise ValueError(f"layer {index}: bad latent-attention sizes")
     elif t == "gla":
         sp.update(tau=float(m["tau"]))
@@ -335,6 +402,14 @@ def layer_spec_params(h: int, sp: dict) -> int:
         m = sp["maps"]
         n = h * m * D * (H + sp["kv_heads"]) + h * sp["kv_heads"] * Dv + H * Dv * h + h
         n += 2 * H if m == 1 else 6 * D + h * H * Dv
+    elif sp["type"] == "sloped_attention":
+        n = h * D * (H + sp["kv_heads"]) + 2 * D + H * Dv * h
+    elif sp["type"] == "delta":
+        c = 2 * sp["kv_heads"] * D + H * Dv
+        n = h * (c + H * Dv + 2 * H) + c * sp["taps"] + 2 * H + Dv + H * Dv * h
+    elif sp["type"] == "latent_attention" and not sp["q_rank"]:
+        R, rd = sp["kv_rank"], sp["rot_dim"]
+        n = h * (H * (D + rd) + R + rd) + R + R * H * (D + Dv) + H + H * Dv * h
     elif sp["type"] == "latent_attention":
         R, Q, rd = sp["kv_rank"], sp["q_rank"], sp["rot_dim"]
         n = h * (Q + R + rd + H) + Q + R + Q * H * (D + rd) + R * H * (D + Dv) + H * Dv * h
@@ -345,7 +420,7 @@ def layer_spec_params(h: int, sp: dict) -> int:
         if f["kind"] == "glu":
             n += 3 * h * f["ff"] + 2 * f["ff"] + h
         else:
-            n += 2 * h * f["ff"] if f["kind"] == "dense" else f["experts"] * (3 * h * f["ff"] + h)
+            n += 2 * h * f["ff"] if f["kind"] == "dense" else f["experts"] * ((3 if f.get("glu", True) else 2) * h * f["ff"] + h)
     return n + 2 * h
 
 

@@ -1,12 +1,15 @@
 """Model families: Llama-3 (8B/70B), Mixtral 8x7B (MoE), GPT-2 — one shard-aware decoder — and
 Nesizen, a heterogeneous stack of attention / gated-linear-attention layers (models/nesizen.py),
 Zinesun, latent-attention layers on a post-norm residual (models/zinesun.py), and Lizizen, parallel
-layers with a token shift over distance-biased and differential attention (models/lizizen.py)."""
+layers with a token shift over distance-biased and differential attention (models/lizizen.py), and
+Gevipel, sandwich-normed layers over sloped window attention, the gated delta rule and latent
+attention with a sink, with routed plain experts (models/gevipel.py)."""
 from .shard import LocalDims, Shard, local_dims  # noqa: F401
 from .transformer import LogicalParam, TransformerLM  # noqa: F401
 from .nesizen import NesizenLM  # noqa: F401
 from .zinesun import ZinesunLM  # noqa: F401
 from .lizizen import LizizenLM  # noqa: F401
+from .gevipel import GevipelLM  # noqa: F401
 
 
 class LlamaForCausalLM(TransformerLM):
@@ -22,7 +25,7 @@ class GPT2LMHeadModel(TransformerLM):
 
 
 _ARCH = {"llama": LlamaForCausalLM, "mixtral": MixtralForCausalLM, "gpt2": GPT2LMHeadModel,
-         "nesizen": NesizenLM, "zinesun": ZinesunLM, "lizizen": LizizenLM}
+         "nesizen": NesizenLM, "zinesun": ZinesunLM, "lizizen": LizizenLM, "gevipel": GevipelLM}
 
 
 def supports_f32(arch: str) -> bool:

@@ -851,7 +851,8 @@ def attn_window_paged(q, k_cache, v_cache, tables, row_cu, positions, scale: flo
 
     Score modifiers, applied in this order before the mask: `q_temp` (coef, every): the scale of a
     row at position p is multiplied by 1 + coef ln(floor((p + 1) / every) + 1); `softcap` > 0:
-    s <- cap tanh(s / cap); `dist_bias` (a, b), f32 [H] each: s <- s - a[h] ln(1 + b[h] (p - j)).
+    s <- cap tanh(s / cap); `dist_bias` (a, b), f32 [H] each: s <- s - a[h] ln(1 + b[h] (p - j)); (a, None):
+    the linear form s <- s - a[h] (p - j).
     `chunk` > 0 replaces the window: a row sees the keys of its own chunk of `chunk` positions
     (counted from position 0). `maps` > 1: the key cache holds `maps` key heads per value head
     (K [blocks, G * maps, BS, D]), the query heads are ordered (head, map), and query head (h, m)
@@ -895,12 +896,13 @@ def gla_out(o, g, norm_w, eps: float, out_dtype):
     return out
 
 
-def moe_route_scores(x, wr, top_k: int, scoring: str = "softmax", renorm: bool = True, bias=None):
+def moe_route_scores(x, wr, top_k: int, scoring: str = "softmax", renorm: bool = True, bias=None, select_bias=None):
     """Router with f32 logits -> (topk_ids [T, k] int32, topk_w [T, k] f32); scoring "softmax" |
     "sigmoid", `renorm`: divide the chosen scores by their sum ("softmax" + renorm = the softmax
-    over the chosen logits alone); `bias` [E] f32 is added to the logits."""
+    over the chosen logits alone); `bias` [E] f32 is added to the logits; `select_bias` [E] f32 is
+    added to the scores for the choice only, the weights being the chosen experts' plain scores."""
     if not _gpu(x):
-        return ref.moe_route_scores(x, wr, top_k, scoring, renorm, bias)
+        return ref.moe_route_scores(x, wr, top_k, scoring, renorm, bias, select_bias)
     T = x.shape[0]
     # logits: a GEMM with f32 accumulation and f32 output (steps of a few rows: one wave per
     # (token, expert) instead of a one-workgroup GEMM), then one wave per token picks
@@ -911,18 +913,22 @@ def moe_route_scores(x, wr, top_k: int, scoring: str = "softmax", renorm: bool =
         logits = linear_act(x, wr, out_dtype=torch.float32)
     ids = _empty(T, top_k, dtype=torch.int32, device=x.device)
     w = _empty(T, top_k, dtype=torch.float32, device=x.device)
-    torch.ops.bfly.moe_topk_scores(logits, bias, top_k, {"softmax": 0, "sigmoid": 1}[scoring], bool(renorm), ids, w)
+    torch.ops.bfly.moe_topk_scores(logits, bias, top_k, {"softmax": 0, "sigmoid": 1}[scoring], bool(renorm), ids, w,
+                                   select_bias)
     return ids, w
 
 
 def moe_glu_ffn(x, topk_ids, topk_w, gate_up_w, down_w, limit: float, alpha: float, up_offset: float = 1.0,
-                scale_input: bool = True):
+                scale_input: bool = True, plain_act=None):
     """Routed GLU experts y = g' sigmoid(alpha g') (u' + up_offset) with g', u' clamped at `limit`
     (inf, alpha 1, up_offset 0: the plain silu GLU). scale_input: each expert runs on (routing
     score * x) and the outputs are summed; otherwise it runs on x and the sum is weighted by the
-    scores. See ops.reference.moe_glu_ffn. gate_up_w [E, 2F, H], down_w [E, H, F]."""
+    scores. See ops.reference.moe_glu_ffn. gate_up_w [E, 2F, H], down_w [E, H, F]. plain_act
+    "relu2": experts without a gate, y = relu(W_up h)^2 with gate_up_w [E, F, H] (limit, alpha and
+    up_offset unused)."""
     if not _gpu(x):
-        return ref.moe_glu_ffn(x, topk_ids, topk_w, gate_up_w, down_w, limit, alpha, None, up_offset, scale_input)
+        return ref.moe_glu_ffn(x, topk_ids, topk_w, gate_up_w, down_w, limit, alpha, None, up_offset, scale_input,
+                               plain_act)
     T, H = x.shape
     E, F = gate_up_w.shape[0], down_w.shape[2]
     TK = T * topk_ids.shape[1]
@@ -933,7 +939,7 @@ def moe_glu_ffn(x, topk_ids, topk_w, gate_up_w, down_w, limit: float, alpha: flo
     y = _arena.get(dev, "moe_glu_y", TK * H, torch.float32)
     out = _empty(T, H, dtype=x.dtype, device=dev)
     torch.ops.bfly.moe_glu_ffn(x, topk_ids, topk_w, gate_up_w, down_w, float(limit), float(alpha), float(up_offset),
-                               bool(scale_input), work, hmid, y, out)
+                               bool(scale_input), work, hmid, y, out, ACTS[plain_act or "none"])
     return out
 
 
@@ -1001,15 +1007,16 @@ def post_norm_add_avg(x, y, norm_w, norm_b, eps: float, scale, stack, index: int
 def latent_prep(z, q_rank: int, kv_rank: int, rot_dim: int, heads: int, qn_w, kvn_w, eps: float, positions, inv_freq,
                 slots, k_cache, v_cache, out_dtype):
     """Rows of z = [query latent | key/value latent | shared rotated key part | gate logits] ->
-    (RMS-normed query latent [T, q_rank], sigmoid gates [T, heads] f32); the normed key/value
+    (RMS-normed query latent [T, q_rank], sigmoid gates [T, heads] f32; q_rank 0 / heads 0: z has no
+    such part and None stands in its place); the normed key/value
     latent and the rotated key part are appended to the paged caches K [blocks, 1, BS, kv_rank +
     rot_dim], V [blocks, 1, kv_rank, BS]."""
     if not _gpu(z):
         return ref.latent_prep(z, q_rank, kv_rank, rot_dim, heads, qn_w, kvn_w, eps, positions, inv_freq, slots,
                                k_cache, v_cache, out_dtype)
     T = z.shape[0]
-    cq = _empty(T, q_rank, dtype=out_dtype, device=z.device)
-    gate = _empty(T, heads, dtype=torch.float32, device=z.device)
+    cq = _empty(T, q_rank, dtype=out_dtype, device=z.device) if q_rank else None
+    gate = _empty(T, heads, dtype=torch.float32, device=z.device) if heads else None
     torch.ops.bfly.latent_prep(z, int(q_rank), int(kv_rank), int(rot_dim), int(heads), qn_w, kvn_w, float(eps), positions,
                                inv_freq, slots, k_cache, v_cache, cq, gate)
     return cq, gate
@@ -1180,3 +1187,57 @@ def _glu_fused_ok(M: int, N: int, K: int) -> bool:
     if ok is None:
         ok = _glu_ok[(M, N, K)] = torch.ops.bfly.gemm_check(M, N, K, EPILOGUES["glu"]) == 0
     return ok
+
+
+# ---------------------------------------------------------------------------------------
+# Sandwich-norm residual stacks with a gated delta rule (csrc/kernels/delta.hip)
+# ---------------------------------------------------------------------------------------
+def post_norm_add_norm(x, y, norm_w, norm_b, eps: float, mult: float, extra, norm2_w, norm2_b, out_dtype):
+    """One launch between two sublayers of a stack with norms on both sides of every sublayer:
+    x <- x + mult * layer_norm(y; norm_w, norm_b) (+ extra [T, W] f32, e.g. the embedding output
+    re-entering before a repeated span), in place in f32, and the next sublayer's input
+    layer_norm(x; norm2_w, norm2_b) in out_dtype (norm2_w None: no next input, returns None)."""
+    if not _gpu(x):
+        return ref.post_norm_add_norm(x, y, norm_w, norm_b, eps, mult, extra, norm2_w, norm2_b, out_dtype)
+    h = None if norm2_w is None else _empty(x.shape[0], x.shape[1], dtype=out_dtype, device=x.device)
+    torch.ops.bfly.post_norm_add_norm(x, y, norm_w, norm_b, float(eps), float(mult), extra, norm2_w, norm2_b, h)
+    return h
+
+
+CONV_ACTS = {"none": 0, "silu": 1}
+
+
+def short_conv_act(z, w, state, state_slots, row_cu, positions, act: str = "silu", out_dtype=torch.float32):
+    """y_t = act(sum_j w[:, j] z_(t - taps + 1 + j)): a short causal convolution over the rows of each
+    sequence of a packed step, per channel, with an activation. z [T, C] may be a view into wider
+    projected rows (any element type the model runs in); w [C, taps] f32, the last column weighs the
+    current row; rows before a sequence's first row of the step come from state[slot] ([slots,
+    taps - 1, C] f32, oldest first) and are zero before position 0. The state is not changed
+    (short_conv_state_update_ does that, after every reader of the old state)."""
+    if not _gpu(z):
+        return ref.short_conv_act(z, w, state, state_slots, row_cu, positions, act, out_dtype)
+    out = _empty(z.shape[0], z.shape[1], dtype=out_dtype, device=z.device)
+    torch.ops.bfly.short_conv_act(z, w, state, state_slots, row_cu, positions, CONV_ACTS[act], out)
+    return out
+
+
+def short_conv_state_update_(z, state, state_slots, row_cu, positions):
+    """state[slot] <- the last taps - 1 rows of z of every sequence of the step (older ones shift)."""
+    if not _gpu(z):
+        return ref.short_conv_state_update_(z, state, state_slots, row_cu, positions)
+    torch.ops.bfly.short_conv_state_update(z, state, state_slots, row_cu, positions)
+    return state
+
+
+def delta_scan(q, k, v, b, a, a_log, dt_bias, state, state_slots, row_cu, positions, q_scale: float,
+               unit_eps: float = 1e-6):
+    """Gated delta rule over packed rows with the state pooled in `state` [slots, H, D, Dv] f32
+    (updated in place; a sequence whose step starts at position 0 starts from zero). q, k [T, G, D],
+    v [T, H, Dv] (views allowed); b, a [T, H] the logits of the write strength and the decay's step;
+    a_log, dt_bias [H] f32. See ops.reference.delta_scan. Returns o [T, H, Dv] f32."""
+    if not _gpu(q):
+        return ref.delta_scan(q, k, v, b, a, a_log, dt_bias, state, state_slots, row_cu, positions, q_scale, unit_eps)
+    o = _empty(q.shape[0], v.shape[1], v.shape[2], dtype=torch.float32, device=q.device)
+    torch.ops.bfly.delta_scan(q, k, v, b, a, a_log, dt_bias, state, state_slots, row_cu, positions, float(q_scale),
+                              float(unit_eps), o)
+    return o

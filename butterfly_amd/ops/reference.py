@@ -631,7 +631,8 @@ def attn_window_paged(q, k_cache, v_cache, tables, row_cu, positions, scale, win
     output is multiplied by its entry (an output gate). chunk > 0: instead of the window, the
     keys of the row's own chunk of `chunk` positions (j >= p - p % chunk). q_temp (coef, every):
     the score is multiplied by 1 + coef ln(floor((p + 1) / every) + 1); softcap > 0: s <- cap
-    tanh(s / cap); dist_bias (a, b) [H] f32: s <- s - a[h] ln(1 + b[h] (p - j)), in that order.
+    tanh(s / cap); dist_bias (a, b) [H] f32: s <- s - a[h] ln(1 + b[h] (p - j)), or with b None the
+    linear form s <- s - a[h] (p - j), in that order.
     maps > 1: the key cache holds `maps` key heads per value head, and query head h reads key
     head ((h / maps) / R) * maps + h % maps (R query-head groups per value head) and its value
     head."""
@@ -665,7 +666,9 @@ def attn_window_paged(q, k_cache, v_cache, tables, row_cu, positions, scale, win
             sc = (qs[:, h] @ K[gk].t()) * rs
             if softcap > 0:
                 sc = softcap * torch.tanh(sc / softcap)
-            if dist_bias is not None:
+            if dist_bias is not None and dist_bias[1] is None:
+                sc = sc - dist_bias[0][h].float() * (p - j).clamp(min=0).float()
+            elif dist_bias is not None:
                 sc = sc - dist_bias[0][h].float() * torch.log1p(dist_bias[1][h].float() * (p - j).clamp(min=0).float())
             sc = sc.masked_fill(~ok, float("-inf"))
             if sink is None:
@@ -713,27 +716,34 @@ def gla_out(o, g, norm_w, eps, out_dtype):
     return (y.reshape(T, H * Dv) * F.silu(g.float())).to(out_dtype)
 
 
-def moe_route_scores(x, wr, top_k, scoring="softmax", renorm=True, bias=None):
+def moe_route_scores(x, wr, top_k, scoring="softmax", renorm=True, bias=None, select_bias=None):
     """Router in f32. scoring "softmax" | "sigmoid"; the top_k largest scores are chosen (ties:
     lowest expert id); `renorm`: the chosen scores are divided by their sum (with "softmax" that
-    is the softmax over the chosen logits alone). `bias` [E] f32 is added to the logits."""
+    is the softmax over the chosen logits alone). `bias` [E] f32 is added to the logits;
+    `select_bias` [E] f32 is added to the scores for the choice only (the weights are the plain
+    scores of the chosen experts)."""
     logits = x.float() @ wr.float().t()
     if bias is not None:
         logits = logits + bias.float()
     sc = torch.softmax(logits, -1) if scoring == "softmax" else torch.sigmoid(logits)
-    w, ids = torch.topk(sc, top_k, -1)
+    if select_bias is not None:
+        ids = torch.topk(sc + select_bias.float(), top_k, -1).indices
+        w = torch.gather(sc, 1, ids)
+    else:
+        w, ids = torch.topk(sc, top_k, -1)
     if renorm:
         w = w / w.sum(-1, keepdim=True)
     return ids.to(torch.int32), w.contiguous()
 
 
 def moe_glu_ffn(x, topk_ids, topk_w, gate_up_w, down_w, limit, alpha, out_dtype=None, up_offset=1.0,
-                scale_input=True):
+                scale_input=True, plain_act=None):
     """Routed GLU experts: g = min(Wg h, limit), u = clamp(Wu h, -limit, limit),
     y = g sigmoid(alpha g) (u + up_offset), output Wd y (limit inf, alpha 1, up_offset 0: the plain
     silu GLU). scale_input: the expert runs on h = w * x and a token's expert outputs are summed;
     otherwise it runs on x and the sum is weighted by w (f32). gate_up_w [E, 2F, H] (gate rows,
-    then up rows), down_w [E, H, F]."""
+    then up rows), down_w [E, H, F]. plain_act "relu2": experts without a gate, y = relu(Wu h)^2
+    with gate_up_w [E, F, H]."""
     T, H = x.shape
     Fd = down_w.shape[2]
     out = torch.zeros(T, H, dtype=torch.float32, device=x.device)
@@ -745,9 +755,13 @@ def moe_glu_ffn(x, topk_ids, topk_w, gate_up_w, down_w, limit, alpha, out_dtype=
             wj = topk_w[tok, j:j + 1].float()
             h = (x[tok].float() * wj).to(x.dtype).float() if scale_input else x[tok].float()
             gu = h @ gate_up_w[e].float().t()
-            g = gu[:, :Fd].clamp(max=limit)
-            u = gu[:, Fd:].clamp(-limit, limit)
-            y = (g * torch.sigmoid(alpha * g) * (u + up_offset)).to(x.dtype).float()
+            if plain_act is not None:
+                assert plain_act == "relu2"
+                y = torch.relu(gu).pow(2).to(x.dtype).float()
+            else:
+                g = gu[:, :Fd].clamp(max=limit)
+                u = gu[:, Fd:].clamp(-limit, limit)
+                y = (g * torch.sigmoid(alpha * g) * (u + up_offset)).to(x.dtype).float()
             yd = y @ down_w[e].float().t()
             out[tok] += yd if scale_input else wj * yd
     return out.to(out_dtype or x.dtype)
@@ -837,13 +851,14 @@ def post_norm_add_avg(x, y, norm_w, norm_b, eps, scale, stack, index, avg_w):
 def latent_prep(z, q_rank, kv_rank, rot_dim, heads, qn_w, kvn_w, eps, positions, inv_freq, slots, k_cache, v_cache,
                 out_dtype):
     """z [T, >= q_rank + kv_rank + rot_dim + heads] holds per row [query latent | key/value latent
-    | shared rotated key part | gate logits]. Returns (RMS-normed query latent [T, q_rank]
+    | shared rotated key part | gate logits] (q_rank 0: no query latent, heads 0: no gates; the
+    result is None in its place). Returns (RMS-normed query latent [T, q_rank]
     out_dtype, sigmoid(gate logits) [T, heads] f32) and appends [normed latent | rotated key part]
     to K [blocks, 1, BS, kv_rank + rot_dim] and the normed latent to V [blocks, 1, kv_rank, BS]."""
     zf = z.float()
     o1, o2, o3 = q_rank, q_rank + kv_rank, q_rank + kv_rank + rot_dim
     rms = lambda u, w: u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) * w.float()  # noqa: E731
-    cq = rms(zf[:, :o1], qn_w).to(out_dtype)
+    cq = rms(zf[:, :o1], qn_w).to(out_dtype) if q_rank else None
     c = rms(zf[:, o1:o2], kvn_w)
     kr = zf[:, o2:o3]
     n = inv_freq.numel()
@@ -852,7 +867,7 @@ def latent_prep(z, q_rank, kv_rank, rot_dim, heads, qn_w, kvn_w, eps, positions,
         cs, sn = torch.cos(a), torch.sin(a)
         u, w = kr[:, 0:2 * n:2], kr[:, 1:2 * n:2]
         kr = torch.cat([torch.stack([u * cs - w * sn, w * cs + u * sn], -1).flatten(-2), kr[:, 2 * n:]], 1)
-    gate = torch.sigmoid(zf[:, o3:o3 + heads]).contiguous()
+    gate = torch.sigmoid(zf[:, o3:o3 + heads]).contiguous() if heads else None
     bs = k_cache.shape[2]
     ok = slots >= 0
     sl = slots[ok].long()
@@ -986,3 +1001,82 @@ def glu_clamp(gu, limit, alpha, up_offset, out_dtype=None, group=0):
     g = g.float().clamp(max=limit)
     u = u.float().clamp(min=-limit, max=limit)
     return (g * torch.sigmoid(alpha * g) * (u + up_offset)).to(out_dtype or gu.dtype)
+
+
+# ---------------------------------------------------------------------------------------
+# Sandwich-norm residual stacks with a gated delta rule: layer norms before and after every
+# sublayer, short causal convolutions with an activation on projected rows, the delta-rule
+# recurrence with pooled per-sequence state.
+# ---------------------------------------------------------------------------------------
+def post_norm_add_norm(x, y, norm_w, norm_b, eps, mult, extra, norm2_w, norm2_b, out_dtype):
+    """x <- x + mult * layer_norm(y; norm_w, norm_b) (+ extra), in place, f32; returns layer_norm(x;
+    norm2_w, norm2_b) in out_dtype, the next sublayer's input (norm2_w None: nothing)."""
+    v = x + mult * _layer_norm_f32(y, norm_w, norm_b, eps)
+    if extra is not None:
+        v = v + extra.float()
+    x.copy_(v)
+    return None if norm2_w is None else _layer_norm_f32(x, norm2_w, norm2_b, eps).to(out_dtype)
+
+
+def short_conv_act(z, w, state, state_slots, row_cu, positions, act, out_dtype):
+    """y_t = act(sum_j w[:, j] z_(t - taps + 1 + j)) per channel over the rows of each sequence of a
+    packed step. z [T, C] (a view of projected rows, any element type); w [C, taps] f32, the last
+    column the current row's; rows before the step's first come from state[slot] ([slots, taps - 1,
+    C] f32, oldest first) and are zero before position 0. act "none" | "silu". The state is not changed."""
+    T, C = z.shape
+    taps = w.shape[1]
+    zf = z.float()
+    y = torch.zeros(T, C, dtype=torch.float32, device=z.device)
+    cu, pos = row_cu.tolist(), positions.tolist()
+    sl = state_slots.tolist() if state_slots is not None else [-1] * (len(cu) - 1)
+    for s in range(len(cu) - 1):
+        a, b = cu[s], cu[s + 1]
+        if b <= a:
+            continue
+        p0 = pos[a]
+        hist = state[sl[s]].clone() if (taps > 1 and sl[s] >= 0) else zf.new_zeros(max(taps - 1, 0), C)
+        for d in range(1, taps):           # hist[taps - 1 - d] is the input d steps before row a
+            if p0 - d < 0:
+                hist[taps - 1 - d] = 0
+        ext = torch.cat([hist, zf[a:b]], 0)
+        for j in range(taps):
+            y[a:b] += w[:, j].float() * ext[j:j + (b - a)]
+    if act == "silu":
+        y = F.silu(y)
+    return y.to(out_dtype)
+
+
+def short_conv_state_update_(z, state, state_slots, row_cu, positions):
+    """After a step: state[slot] holds the last taps - 1 rows of z of every sequence (oldest first)."""
+    return conv_state_update_(z.float(), state, state_slots, row_cu, positions)
+
+
+def delta_scan(q, k, v, b, a, a_log, dt_bias, state, state_slots, row_cu, positions, q_scale, unit_eps):
+    """Gated delta rule over packed rows, all f32. q, k [T, G, D] and v [T, H, Dv] (head h reads
+    query / key group h // (H / G)); q and k are first made unit vectors, x / sqrt(sum x^2 +
+    unit_eps), and q is multiplied by q_scale. Per row and head: beta = sigmoid(b), decay =
+    exp(-exp(a_log[h]) softplus(a + dt_bias[h])); S <- decay S; u = beta (v - S^T k); S <- S + k u^T;
+    o = S^T q. The state S [D, Dv] of sequence s is read from state[state_slots[s]] unless its first
+    row is at position 0 (then zero) and written back after its last row. Returns o [T, H, Dv] f32."""
+    T, G, D = q.shape
+    H, Dv = v.shape[1], v.shape[2]
+    rep = H // G
+    qf, kf, vf = q.float(), k.float(), v.float()
+    qf = qf * torch.rsqrt(qf.pow(2).sum(-1, keepdim=True) + unit_eps) * q_scale
+    kf = kf * torch.rsqrt(kf.pow(2).sum(-1, keepdim=True) + unit_eps)
+    qf, kf = qf.repeat_interleave(rep, 1), kf.repeat_interleave(rep, 1)
+    beta = torch.sigmoid(b.float())
+    decay = torch.exp(-torch.exp(a_log.float()) * F.softplus(a.float() + dt_bias.float()))
+    o = torch.zeros(T, H, Dv, dtype=torch.float32, device=q.device)
+    cu, pos, sl = row_cu.tolist(), positions.tolist(), state_slots.tolist()
+    for s in range(len(cu) - 1):
+        if cu[s + 1] == cu[s] or sl[s] < 0:
+            continue
+        S = torch.zeros(H, D, Dv, dtype=torch.float32, device=q.device) if pos[cu[s]] == 0 else state[sl[s]].clone()
+        for t in range(cu[s], cu[s + 1]):
+            S = decay[t][:, None, None] * S
+            u = beta[t][:, None] * (vf[t] - torch.einsum("hdv,hd->hv", S, kf[t]))
+            S = S + kf[t][:, :, None] * u[:, None, :]
+            o[t] = torch.einsum("hdv,hd->hv", S, qf[t])
+        state[sl[s]] = S
+    return o
