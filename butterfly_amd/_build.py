@@ -28,7 +28,7 @@ PKG = ROOT / "butterfly_amd"
 CSRC = ROOT / "csrc"
 OBJ = ROOT / "build" / "obj"
 ARCH = os.environ.get("BFLY_OFFLOAD_ARCH", "gfx950")
-PRECISE_KERNELS = {"gemm_any", "hyper", "mixers", "postnorm", "parlayer"}
+PRECISE_KERNELS = {"gemm_any", "hyper", "mixers", "postnorm", "parlayer", "delta"}
 HIPCC = os.environ.get("HIPCC", shutil.which("hipcc") or "/opt/rocm/bin/hipcc")
 
 

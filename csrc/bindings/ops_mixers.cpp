@@ -196,12 +196,16 @@ void attn_window_paged(const Tensor& q, const Tensor& k_cache, const Tensor& v_c
   CHK_I32(row_cu);
   TORCH_CHECK(row_cu.numel() == tables.size(0) + 1, "attn_window_paged: row_cu");
   TORCH_CHECK(G > 0 && H % (G * maps) == 0 && Dv <= 512 && D <= 4096, "attn_window_paged: head counts / sizes");
-  TORCH_CHECK(dist_a.has_value() == dist_b.has_value(), "attn_window_paged: the distance bias needs both vectors");
-  if (dist_a.has_value()) {
-    CHK_F32(*dist_a); CHK_F32(*dist_b);
-    TORCH_CHECK(dist_a->numel() == H && dist_b->numel() == H, "attn_window_paged: distance bias [H]");
+  TORCH_CHECK(dist_a.has_value() || !dist_b.has_value(), "attn_window_paged: dist_b needs dist_a");
+  if (dist_a.has_value()) {      // (a, b): logarithmic, a alone: linear
+    CHK_F32(*dist_a);
+    TORCH_CHECK(dist_a->is_cuda() && dist_a->numel() == H, "attn_window_paged: distance bias [H]");
     md.dist_a = dist_a->data_ptr<float>();
-    md.dist_b = dist_b->data_ptr<float>();
+    if (dist_b.has_value()) {
+      CHK_F32(*dist_b);
+      TORCH_CHECK(dist_b->is_cuda() && dist_b->numel() == H, "attn_window_paged: distance bias [H]");
+      md.dist_b = dist_b->data_ptr<float>();
+    }
   }
   TORCH_CHECK(tables.dim() == 2 && row_seq_t.numel() == T && positions.numel() == T, "attn_window_paged: index shapes");
   const float *sinkp = nullptr, *gatep = nullptr;
@@ -280,7 +284,7 @@ void router_logits(const Tensor& x, const Tensor& wr, Tensor& logits) {
 }
 
 void moe_topk_scores(const Tensor& logits, const optional<Tensor>& bias, int64_t top_k, int64_t scoring, bool renorm,
-                     Tensor& ids, Tensor& w) {
+                     Tensor& ids, Tensor& w, const optional<Tensor>& select_bias) {
   CHK_GPU(logits); CHK_F32(logits); CHK_I32(ids); CHK_F32(w);
   const float* bp = nullptr;
   if (bias.has_value()) {
@@ -288,12 +292,18 @@ void moe_topk_scores(const Tensor& logits, const optional<Tensor>& bias, int64_t
     TORCH_CHECK(bias->numel() == logits.size(1), "moe_topk_scores: bias [E]");
     bp = bias->data_ptr<float>();
   }
+  const float* sbp = nullptr;
+  if (select_bias.has_value()) {
+    CHK_F32(*select_bias);
+    TORCH_CHECK(select_bias->is_cuda() && select_bias->numel() == logits.size(1), "moe_topk_scores: select_bias [E]");
+    sbp = select_bias->data_ptr<float>();
+  }
   TORCH_CHECK(logits.dim() == 2, "moe_topk_scores: logits [T, E]");
   const int64_t T = logits.size(0), E = logits.size(1);
   TORCH_CHECK(E >= 1 && E <= 1024 && top_k >= 1 && top_k <= E, "moe_topk_scores: experts / top_k");
   TORCH_CHECK(ids.numel() == T * top_k && w.numel() == T * top_k, "moe_topk_scores: outputs");
   bfly::launch_moe_topk_scores(logits.data_ptr<float>(), bp, (int)top_k, (int)scoring, renorm, ids.data_ptr<int>(),
-                               w.data_ptr<float>(), (int)T, (int)E, cur_stream());
+                               w.data_ptr<float>(), (int)T, (int)E, cur_stream(), sbp);
 }
 
 int64_t moe_sort_max_tiles(int64_t TK, int64_t E) { return bfly::moe_sort_max_tiles((int)TK, (int)E); }
@@ -301,7 +311,7 @@ int64_t moe_sort_max_tiles(int64_t TK, int64_t E) { return bfly::moe_sort_max_ti
 // work: int32 [TK + (E + 1) + 2 * max_tiles + 1] = perm | offsets | tiles | ntiles
 void moe_glu_ffn(const Tensor& x, const Tensor& topk_ids, const Tensor& topk_w, const Tensor& gate_up_w,
                  const Tensor& down_w, double limit, double alpha, double up_offset, bool scale_input, Tensor& work,
-                 Tensor& hmid, Tensor& y, Tensor& out) {
+                 Tensor& hmid, Tensor& y, Tensor& out, int64_t plain_act) {
   CHK_GPU(x); CHK_SAME(x, gate_up_w); CHK_SAME(x, down_w); CHK_SAME(x, hmid); CHK_SAME(x, out);
   CHK_I32(topk_ids); CHK_F32(topk_w); CHK_I32(work); CHK_F32(y);
   TORCH_CHECK(x.dim() == 2 && x.stride(1) == 1 && gate_up_w.dim() == 3 && down_w.dim() == 3 &&
@@ -309,8 +319,10 @@ void moe_glu_ffn(const Tensor& x, const Tensor& topk_ids, const Tensor& topk_w, 
   const int64_t T = x.size(0), Hd = x.size(1), E = gate_up_w.size(0), F = down_w.size(2);
   TORCH_CHECK(topk_ids.dim() == 2 && topk_ids.size(0) == T && topk_w.numel() == topk_ids.numel(), "moe_glu_ffn: routing");
   const int64_t K = topk_ids.size(1), TK = T * K;
-  TORCH_CHECK(E <= 1024 && gate_up_w.size(1) == 2 * F && gate_up_w.size(2) == Hd && down_w.size(0) == E &&
-                  down_w.size(1) == Hd, "moe_glu_ffn: weights [E, 2F, H] / [E, H, F]");
+  TORCH_CHECK(plain_act == bfly::ACT_NONE || plain_act == bfly::ACT_RELU2, "moe_glu_ffn: plain experts take relu2");
+  TORCH_CHECK(E <= 1024 && gate_up_w.size(1) == (plain_act ? F : 2 * F) && gate_up_w.size(2) == Hd &&
+                  down_w.size(0) == E && down_w.size(1) == Hd,
+              "moe_glu_ffn: weights [E, 2F, H] (plain experts: [E, F, H]) / [E, H, F]");
   const int64_t mt = bfly::moe_sort_max_tiles((int)TK, (int)E);
   TORCH_CHECK(work.numel() >= TK + E + 1 + 2 * mt + 1, "moe_glu_ffn: work buffer");
   TORCH_CHECK(hmid.is_contiguous() && hmid.numel() >= TK * F && y.numel() >= TK * Hd && out.is_contiguous() &&
@@ -327,7 +339,7 @@ void moe_glu_ffn(const Tensor& x, const Tensor& topk_ids, const Tensor& topk_w, 
   // scores on the expert's input (the row is scaled and the outputs are summed) or on its output
   bfly::launch_moe_glu_up(x.data_ptr(), x.stride(0), scale_input ? topk_w.data_ptr<float>() : nullptr, (int)K, perm,
                           offsets, tiles, ntiles, (int)mt, gate_up_w.data_ptr(), (float)limit, (float)alpha,
-                          (float)up_offset, hmid.data_ptr(), (int)Hd, (int)F, f32, tr, s);
+                          (float)up_offset, hmid.data_ptr(), (int)Hd, (int)F, f32, tr, s, (int)plain_act);
   bfly::launch_moe_down(hmid.data_ptr(), perm, offsets, tiles, ntiles, (int)mt, down_w.data_ptr(), y.data_ptr<float>(),
                         (int)Hd, (int)F, f32, tr, s);
   bfly::launch_moe_sum(y.data_ptr<float>(), scale_input ? nullptr : topk_w.data_ptr<float>(), (int)K, out.data_ptr(),
@@ -368,11 +380,11 @@ TORCH_LIBRARY_FRAGMENT(bfly, m) {
   m.def("gla_out(Tensor o, Tensor g, Tensor norm_w, float eps, Tensor(a!) out) -> ()");
   m.def("router_logits(Tensor x, Tensor wr, Tensor(a!) logits) -> ()");
   m.def("moe_topk_scores(Tensor logits, Tensor? bias, int top_k, int scoring, bool renorm, Tensor(a!) ids, "
-        "Tensor(b!) w) -> ()");
+        "Tensor(b!) w, Tensor? select_bias=None) -> ()");
   m.def("moe_sort_max_tiles(int tk, int experts) -> int", &moe_sort_max_tiles);
   m.def("moe_glu_ffn(Tensor x, Tensor topk_ids, Tensor topk_w, Tensor gate_up_w, Tensor down_w, float limit, "
         "float alpha, float up_offset, bool scale_input, Tensor(a!) work, Tensor(b!) hmid, Tensor(c!) y, "
-        "Tensor(d!) out) -> ()");
+        "Tensor(d!) out, int plain_act=0) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(bfly, CUDA, m) {

@@ -108,28 +108,35 @@ void post_norm_add_avg(Tensor& x, const optional<Tensor>& y, const optional<Tens
                                  (int)index, avg.data_ptr<float>(), (int)T, (int)W, f32, cur_stream());
 }
 
-void latent_prep(const Tensor& z, int64_t Q, int64_t R, int64_t rd, int64_t H, const Tensor& qn_w, const Tensor& kvn_w,
-                 double eps, const Tensor& positions, const Tensor& inv_freq, const Tensor& slots, Tensor& k_cache,
-                 Tensor& v_cache, Tensor& cq, Tensor& gate) {
-  CHK_GPU(z); CHK_F32(qn_w); CHK_F32(kvn_w); CHK_I32(positions); CHK_F32(inv_freq); CHK_I32(slots); CHK_F32(gate);
-  CHK_SAME(k_cache, z); CHK_SAME(v_cache, z); CHK_SAME(cq, z);
-  TORCH_CHECK(z.dim() == 2 && z.stride(1) == 1 && Q >= 1 && R >= 1 && rd >= 0 && H >= 0 && z.size(1) >= Q + R + rd + H,
+void latent_prep(const Tensor& z, int64_t Q, int64_t R, int64_t rd, int64_t H, const optional<Tensor>& qn_w,
+                 const Tensor& kvn_w, double eps, const Tensor& positions, const Tensor& inv_freq, const Tensor& slots,
+                 Tensor& k_cache, Tensor& v_cache, const optional<Tensor>& cq, const optional<Tensor>& gate) {
+  CHK_GPU(z); CHK_F32(kvn_w); CHK_I32(positions); CHK_F32(inv_freq); CHK_I32(slots);
+  CHK_SAME(k_cache, z); CHK_SAME(v_cache, z);
+  TORCH_CHECK(z.dim() == 2 && z.stride(1) == 1 && Q >= 0 && R >= 1 && rd >= 0 && H >= 0 && z.size(1) >= Q + R + rd + H,
               "latent_prep: z [T, >= Q + R + rd + H]");
   const int64_t T = z.size(0);
-  TORCH_CHECK(qn_w.numel() == Q && kvn_w.numel() == R && positions.numel() == T && slots.numel() == T &&
+  // Q == 0: no query latent (no weight, no output); H == 0: no gates
+  TORCH_CHECK((Q > 0) == qn_w.has_value() && (Q > 0) == cq.has_value() && (H > 0) == gate.has_value(),
+              "latent_prep: the query latent needs its norm weight and output, the gates their output");
+  if (Q > 0) { CHK_F32(*qn_w); CHK_SAME(*cq, z); TORCH_CHECK(qn_w->numel() == Q, "latent_prep: query norm weight [Q]"); }
+  if (H > 0) CHK_F32(*gate);
+  TORCH_CHECK(kvn_w.numel() == R && positions.numel() == T && slots.numel() == T &&
                   2 * inv_freq.numel() <= rd, "latent_prep: norm weights / positions / slots / frequencies");
   TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.is_contiguous() && v_cache.is_contiguous() &&
                   k_cache.size(1) == 1 && v_cache.size(1) == 1 && k_cache.size(3) >= R + rd && v_cache.size(2) >= R &&
                   v_cache.size(3) == k_cache.size(2) && v_cache.size(0) == k_cache.size(0),
               "latent_prep: caches K [blocks, 1, BS, >= R + rd], V [blocks, 1, >= R, BS]");
-  TORCH_CHECK(cq.is_contiguous() && cq.dim() == 2 && cq.size(0) == T && cq.size(1) == Q && gate.numel() == T * H,
-              "latent_prep: outputs");
+  TORCH_CHECK((Q == 0 || (cq->is_contiguous() && cq->dim() == 2 && cq->size(0) == T && cq->size(1) == Q)) &&
+                  (H == 0 || gate->numel() == T * H), "latent_prep: outputs");
   // slots are produced by the block manager for this cache: blocks * BS bounds them
-  bfly::launch_latent_prep(z.data_ptr(), z.stride(0), (int)Q, (int)R, (int)rd, (int)H, qn_w.data_ptr<float>(),
+  bfly::launch_latent_prep(z.data_ptr(), z.stride(0), (int)Q, (int)R, (int)rd, (int)H,
+                           Q > 0 ? qn_w->data_ptr<float>() : nullptr,
                            kvn_w.data_ptr<float>(), (float)eps, positions.data_ptr<int>(), inv_freq.data_ptr<float>(),
                            (int)inv_freq.numel(), slots.data_ptr<int>(), k_cache.data_ptr(), v_cache.data_ptr(),
-                           (int)k_cache.size(2), (int)k_cache.size(3), (int)v_cache.size(2), cq.data_ptr(),
-                           gate.data_ptr<float>(), (int)T, is_f32(z), cur_stream());
+                           (int)k_cache.size(2), (int)k_cache.size(3), (int)v_cache.size(2),
+                           Q > 0 ? cq->data_ptr() : nullptr, H > 0 ? gate->data_ptr<float>() : nullptr, (int)T,
+                           is_f32(z), cur_stream());
 }
 
 void rope_heads_copy(const Tensor& src, Tensor& dst, const Tensor& positions, const Tensor& inv_freq) {
@@ -173,9 +180,9 @@ TORCH_LIBRARY_FRAGMENT(bfly, m) {
         "Tensor(b!)? cast) -> ()");
   m.def("post_norm_add_avg(Tensor(a!) x, Tensor? y, Tensor? nw, Tensor? nb, float eps, Tensor? scale, Tensor(b!) stack, "
         "int index, Tensor avg) -> ()");
-  m.def("latent_prep(Tensor z, int q_rank, int kv_rank, int rot_dim, int heads, Tensor qn_w, Tensor kvn_w, float eps, "
-        "Tensor positions, Tensor inv_freq, Tensor slots, Tensor(a!) k_cache, Tensor(b!) v_cache, Tensor(c!) cq, "
-        "Tensor(d!) gate) -> ()");
+  m.def("latent_prep(Tensor z, int q_rank, int kv_rank, int rot_dim, int heads, Tensor? qn_w, Tensor kvn_w, float eps, "
+        "Tensor positions, Tensor inv_freq, Tensor slots, Tensor(a!) k_cache, Tensor(b!) v_cache, Tensor(c!)? cq, "
+        "Tensor(d!)? gate) -> ()");
   m.def("rope_heads_copy(Tensor src, Tensor(a!) dst, Tensor positions, Tensor inv_freq) -> ()");
   m.def("layer_norm_rows(Tensor x, Tensor nw, Tensor nb, float eps, Tensor? idx, Tensor(a!) out) -> ()");
 }

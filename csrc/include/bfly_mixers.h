@@ -54,7 +54,7 @@ struct AttnMod {
                                   // (j >= p - p % chunk)
   float softcap = 0.f;            // > 0: s <- cap tanh(s / cap)
   const float* dist_a = nullptr;  // [H] (with dist_b): s <- s - a[h] ln(1 + b[h] (p - j))
-  const float* dist_b = nullptr;
+  const float* dist_b = nullptr;  // nullptr with dist_a set: the linear form s <- s - a[h] (p - j)
   float qt_coef = 0.f;            // the score scale of a row at p is multiplied by
   int qt_every = 1;               // 1 + coef ln(floor((p + 1) / every) + 1)
   int maps = 1;                   // key heads per value head: K [blocks, G * maps, BS, D]; query heads are ordered
@@ -96,9 +96,10 @@ void launch_gla_out(const float* o, const void* g, long g_ld, const float* norm_
 void launch_router_logits(const void* x, long ldx, const void* wr, float* logits, int T, int E, int Hd, bool f32,
                           hipStream_t s);
 // Router choice from f32 logits [T, E] (+ bias [E], nullable): scoring 0 softmax / 1 sigmoid, top-k
-// (ties: lowest id), optional renorm. E <= 1024.
+// (ties: lowest id), optional renorm. select_bias [E] (nullable) is added to the scores for the choice
+// only; the weights are the chosen experts' plain scores. E <= 1024.
 void launch_moe_topk_scores(const float* logits, const float* bias, int top_k, int scoring, bool renorm, int* ids,
-                            float* w, int T, int E, hipStream_t s);
+                            float* w, int T, int E, hipStream_t s, const float* select_bias = nullptr);
 // Group the T*K (token, choice) pairs by expert: perm [TK] pair indices grouped by expert,
 // offsets [E + 1], tiles [max_tiles][2] = (expert, first row) of every tile_rows-row tile, ntiles [1].
 void launch_moe_sort(const int* ids, int TK, int E, int* perm, int* offsets, int* tiles, int* ntiles, int tile_rows,
@@ -107,10 +108,12 @@ int moe_sort_max_tiles(int TK, int E);
 // rows per tile of the grouped expert GEMMs for this problem (64, or 128 for large bf16 groups)
 int moe_tile_rows(int TK, int E, bool f32);
 // hmid[r, f] = g' sigmoid(alpha g') (u' + up_offset), (g', u') the clamped gate / up products of
-// expert e(r) on (w x) for grouped row r (topk_w == nullptr: on x itself)
+// expert e(r) on (w x) for grouped row r (topk_w == nullptr: on x itself). plain_act != ACT_NONE: experts
+// without a gate, gate_up_w [E, F, Hd] and hmid = act(up product) (ACT_RELU2)
 void launch_moe_glu_up(const void* x, long ldx, const float* topk_w, int K, const int* perm, const int* offsets,
                        const int* tiles, const int* ntiles, int max_tiles, const void* gate_up_w, float limit,
-                       float alpha, float up_offset, void* hmid, int Hd, int F, bool f32, int tile_rows, hipStream_t s);
+                       float alpha, float up_offset, void* hmid, int Hd, int F, bool f32, int tile_rows, hipStream_t s,
+                       int plain_act = ACT_NONE);
 // y[perm[r], :] = down_e(r) hmid[r]     (y f32, pair order)
 void launch_moe_down(const void* hmid, const int* perm, const int* offsets, const int* tiles, const int* ntiles,
                      int max_tiles, const void* down_w, float* y, int Hd, int F, bool f32, int tile_rows, hipStream_t s);

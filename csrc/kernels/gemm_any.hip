@@ -142,7 +142,8 @@ __global__ __launch_bounds__(256) void moe_glu_up_kernel(const T* __restrict__ x
                                                          const int* __restrict__ perm, const int* __restrict__ offsets_e,
                                                          const int* __restrict__ tiles, const int* __restrict__ ntiles,
                                                          const T* __restrict__ gu_w, float limit, float alpha,
-                                                         float up_offset, T* __restrict__ hmid, int Hd, int F) {
+                                                         float up_offset, T* __restrict__ hmid, int Hd, int F,
+                                                         int plain) {
   if ((int)blockIdx.y >= ntiles[0]) return;
   __shared__ float As[TK][LDP], Bs[TK][LDP];
   __shared__ int tok[TM];
@@ -157,7 +158,8 @@ __global__ __launch_bounds__(256) void moe_glu_up_kernel(const T* __restrict__ x
     wt[threadIdx.x] = p < 0 ? 0.f : (topk_w ? topk_w[p] : 1.f);      // no scores: the row as it is
   }
   __syncthreads();
-  const T* wg = gu_w + (long)e * 2 * F * Hd;
+  // plain experts (no gate): F rows per expert, hmid = act(W x)
+  const T* wg = gu_w + (long)e * (plain ? 1 : 2) * F * Hd;
   const T* wu = wg + (long)F * Hd;
   // the expert's input is the token row times its routing score, rounded to the activation type
   auto la = [&](int r, int k) {
@@ -167,8 +169,9 @@ __global__ __launch_bounds__(256) void moe_glu_up_kernel(const T* __restrict__ x
   float g[4][4] = {}, u[4][4] = {};
   tile_mac(g, la, [&](int c, int k) { return (col0 + c < F && k < Hd) ? ldf(wg + (long)(col0 + c) * Hd + k) : 0.f; },
            Hd, As, Bs);
-  tile_mac(u, la, [&](int c, int k) { return (col0 + c < F && k < Hd) ? ldf(wu + (long)(col0 + c) * Hd + k) : 0.f; },
-           Hd, As, Bs);
+  if (!plain)
+    tile_mac(u, la, [&](int c, int k) { return (col0 + c < F && k < Hd) ? ldf(wu + (long)(col0 + c) * Hd + k) : 0.f; },
+             Hd, As, Bs);
   const int ty = threadIdx.x >> 4, tx = threadIdx.x & 15;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -178,6 +181,10 @@ __global__ __launch_bounds__(256) void moe_glu_up_kernel(const T* __restrict__ x
     for (int j = 0; j < 4; ++j) {
       const int c = col0 + tx * 4 + j;
       if (c >= F) continue;
+      if (plain) {
+        hmid[(long)r * F + c] = cvt<T>(apply_act(g[i][j], plain, 0.f, 0.f));
+        continue;
+      }
       const float gg = fminf(g[i][j], limit);
       const float uu = fminf(fmaxf(u[i][j], -limit), limit);
       const float y = gg / (1.f + expf(-alpha * gg)) * (uu + up_offset);
@@ -254,8 +261,8 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const T* __restrict_
 __global__ __launch_bounds__(64) void moe_topk_scores_kernel(const float* __restrict__ logits,
                                                              const float* __restrict__ bias, int top_k, int scoring,
                                                              int renorm, int* __restrict__ ids, float* __restrict__ w,
-                                                             int E) {
-  __shared__ float sc[1024];
+                                                             int E, const float* __restrict__ sel) {
+  __shared__ float sc[1024], raw[1024];
   const int t = blockIdx.x, lane = threadIdx.x;
   for (int e = lane; e < E; e += 64) sc[e] = logits[(long)t * E + e] + (bias ? bias[e] : 0.f);
   __syncthreads();
@@ -272,6 +279,13 @@ __global__ __launch_bounds__(64) void moe_topk_scores_kernel(const float* __rest
     for (int e = lane; e < E; e += 64) sc[e] = 1.f / (1.f + expf(-sc[e]));
   }
   __syncthreads();
+  if (sel) {      // the choice is made among score + sel; the weight is the plain score
+    for (int e = lane; e < E; e += 64) {
+      raw[e] = sc[e];
+      sc[e] += sel[e];
+    }
+    __syncthreads();
+  }
   float sum = 0.f;
   for (int k = 0; k < top_k; ++k) {
     float bv = -INFINITY;
@@ -286,6 +300,7 @@ __global__ __launch_bounds__(64) void moe_topk_scores_kernel(const float* __rest
       const int oi = __shfl_xor(bi, o, 64);
       if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
     }
+    if (sel && bi < E) bv = raw[bi];
     sum += bv;
     if (lane == 0) {      // (a row of NaN scores selects nothing: id -1)
       const bool ok = bi < E;
@@ -521,7 +536,8 @@ __global__ __launch_bounds__(256) void moe_glu_up_mfma_kernel(const bf16* __rest
                                                               const int* __restrict__ tiles,
                                                               const int* __restrict__ ntiles,
                                                               const bf16* __restrict__ gu_w, float limit, float alpha,
-                                                              float up_offset, bf16* __restrict__ hmid, int Hd, int F) {
+                                                              float up_offset, bf16* __restrict__ hmid, int Hd, int F,
+                                                              int plain) {
   if ((int)blockIdx.y >= ntiles[0]) return;
   constexpr int BT = 32 * WT;
   // small groups (decode): gate and up share one K loop, so both panels' weight segments are in
@@ -531,7 +547,8 @@ __global__ __launch_bounds__(256) void moe_glu_up_mfma_kernel(const bf16* __rest
   const int e = tiles[2 * blockIdx.y], r0 = tiles[2 * blockIdx.y + 1];
   const int rend = offsets_e[e + 1];
   const int col0 = blockIdx.x * BT;
-  const bf16* wg = gu_w + (long)e * 2 * F * Hd;
+  // plain experts (no gate): F rows per expert, hmid = act(W x)
+  const bf16* wg = gu_w + (long)e * (plain ? 1 : 2) * F * Hd;
   const bf16* wu = wg + (long)F * Hd;
   // the expert's input row: the token row times its routing score, rounded to bf16
   auto rowX = [&](int r) {
@@ -542,6 +559,14 @@ __global__ __launch_bounds__(256) void moe_glu_up_mfma_kernel(const bf16* __rest
   BFLY_ZERO_ACC(u);
   auto rowG = [&](int c) { return RowRef{col0 + c < F ? wg + (long)(col0 + c) * Hd : nullptr, 1.f}; };
   auto rowU = [&](int c) { return RowRef{col0 + c < F ? wu + (long)(col0 + c) * Hd : nullptr, 1.f}; };
+  if (plain) {
+    tile_mac_mfma<WT>(g, rowX, rowG, Hd, Xs, Ws);
+    tile_each<WT>(g, [&](int m, int n, float v) {
+      const int r = r0 + m, c = col0 + n;
+      if (r < rend && c < F) hmid[(long)r * F + c] = (bf16)apply_act(v, plain, 0.f, 0.f);
+    });
+    return;
+  }
   if constexpr (WT == 2) {
     tile_mac_mfma2<WT>(g, u, rowX, rowG, rowU, Hd, Xs, Ws, Vs);
   } else {
@@ -633,9 +658,9 @@ void launch_router_logits(const void* x, long ldx, const void* wr, float* logits
 }
 
 void launch_moe_topk_scores(const float* logits, const float* bias, int top_k, int scoring, bool renorm, int* ids,
-                            float* w, int T, int E, hipStream_t s) {
+                            float* w, int T, int E, hipStream_t s, const float* select_bias) {
   if (T <= 0) return;
-  moe_topk_scores_kernel<<<T, 64, 0, s>>>(logits, bias, top_k, scoring, renorm, ids, w, E);
+  moe_topk_scores_kernel<<<T, 64, 0, s>>>(logits, bias, top_k, scoring, renorm, ids, w, E, select_bias);
 }
 
 int moe_sort_max_tiles(int TKp, int E) { return (TKp + 63) / 64 + E; }
@@ -650,20 +675,24 @@ void launch_moe_sort(const int* ids, int TKp, int E, int* perm, int* offsets, in
 
 void launch_moe_glu_up(const void* x, long ldx, const float* topk_w, int K, const int* perm, const int* offsets,
                        const int* tiles, const int* ntiles, int max_tiles, const void* gate_up_w, float limit,
-                       float alpha, float up_offset, void* hmid, int Hd, int F, bool f32, int tile_rows, hipStream_t s) {
+                       float alpha, float up_offset, void* hmid, int Hd, int F, bool f32, int tile_rows, hipStream_t s,
+                       int plain_act) {
   if (tile_rows == 128) {
     dim3 g2((F + 127) / 128, max_tiles);
     moe_glu_up_mfma_kernel<4><<<g2, 256, 0, s>>>((const bf16*)x, ldx, topk_w, K, perm, offsets, tiles, ntiles,
-                                                 (const bf16*)gate_up_w, limit, alpha, up_offset, (bf16*)hmid, Hd, F);
+                                                 (const bf16*)gate_up_w, limit, alpha, up_offset, (bf16*)hmid, Hd, F,
+                                                 plain_act);
     return;
   }
   dim3 grid((F + TN - 1) / TN, max_tiles);
   if (f32)
     moe_glu_up_kernel<float><<<grid, 256, 0, s>>>((const float*)x, ldx, topk_w, K, perm, offsets, tiles, ntiles,
-                                                  (const float*)gate_up_w, limit, alpha, up_offset, (float*)hmid, Hd, F);
+                                                  (const float*)gate_up_w, limit, alpha, up_offset, (float*)hmid, Hd, F,
+                                                  plain_act);
   else
     moe_glu_up_mfma_kernel<2><<<grid, 256, 0, s>>>((const bf16*)x, ldx, topk_w, K, perm, offsets, tiles, ntiles,
-                                                (const bf16*)gate_up_w, limit, alpha, up_offset, (bf16*)hmid, Hd, F);
+                                                (const bf16*)gate_up_w, limit, alpha, up_offset, (bf16*)hmid, Hd, F,
+                                                plain_act);
 }
 
 void launch_moe_down(const void* hmid, const int* perm, const int* offsets, const int* tiles, const int* ntiles,

@@ -85,7 +85,10 @@ __device__ __forceinline__ float attn_score(float dot, float rscale, int dist, f
     if (FAST) sc = md.softcap * (1.f - __fdividef(2.f, __expf(2.f * __fdividef(sc, md.softcap)) + 1.f));
     else sc = md.softcap * tanhf(sc / md.softcap);
   }
-  if (md.dist_a) sc -= da * (FAST ? __logf(1.f + db * (float)dist) : log1pf(db * (float)dist));
+  if (md.dist_a) {      // no second vector: the linear form
+    if (!md.dist_b) sc -= da * (float)dist;
+    else sc -= da * (FAST ? __logf(1.f + db * (float)dist) : log1pf(db * (float)dist));
+  }
   return sc;
 }
 
@@ -123,7 +126,7 @@ __global__ __launch_bounds__(64) void attn_window_paged_kernel(const T* __restri
   }
   const int p = positions[t];
   const float rscale = attn_row_scale(p, scale, md);
-  const float da = md.dist_a ? md.dist_a[h] : 0.f, db = md.dist_a ? md.dist_b[h] : 0.f;
+  const float da = md.dist_a ? md.dist_a[h] : 0.f, db = md.dist_b ? md.dist_b[h] : 0.f;
   const int* tab = tables + (long)s * max_blocks;
   for (int d = lane; d < D; d += 64) sq[d] = (float)q[t * q_ld + (long)h * D + d];
   __syncthreads();
@@ -233,7 +236,7 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __res
   const int p = rv ? positions[row] : -1;
   const int plo = attn_row_lo(max(p, 0), window, md.chunk);
   const float rscale = attn_row_scale(max(p, 0), scale, md);
-  const float da = md.dist_a ? md.dist_a[h] : 0.f, db = md.dist_a ? md.dist_b[h] : 0.f;
+  const float da = md.dist_a ? md.dist_a[h] : 0.f, db = md.dist_b ? md.dist_b[h] : 0.f;
   int pmin = rv ? p : 0x7fffffff, pmax = p;
 #pragma unroll
   for (int o = 1; o < 16; o <<= 1) {

@@ -255,7 +255,7 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(const T* __restrict__ 
   float a = 0.f, b = 0.f;
   for (int i = threadIdx.x; i < Q; i += blockDim.x) { const float v = (float)zr[i]; a = fmaf(v, v, a); }
   for (int i = threadIdx.x; i < R; i += blockDim.x) { const float v = (float)zr[Q + i]; b = fmaf(v, v, b); }
-  const float rq = 1.f / sqrtf(block_sum(a, red) / (float)Q + eps);
+  const float rq = Q > 0 ? 1.f / sqrtf(block_sum(a, red) / (float)Q + eps) : 0.f;     // (Q, H = 0: no query latent, no gates)
   const float rk = 1.f / sqrtf(block_sum(b, red) / (float)R + eps);
   for (int i = threadIdx.x; i < Q; i += blockDim.x) cq[t * Q + i] = (T)((float)zr[i] * rq * qn_w[i]);
   for (int i = threadIdx.x; i < H; i += blockDim.x) gate[t * H + i] = 1.f / (1.f + expf(-(float)zr[Q + R + rd + i]));
