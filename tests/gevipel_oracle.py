@@ -163,29 +163,39 @@ def delta_mixer(h, m, w, p, eps):
     return o.reshape(T, H * Dv) @ w[p + "o"].T
 
 
+def sloped_window_softmax(q, k, v, scale, window, q_temp):
+    """q [T, H, D], k, v [T, G, D]: softmax attention of position i over the keys j with 0 <= i - j < window
+    (None: all j <= i); the score of head h loses 2^(-8 (h + 1) / H) (i - j); q_temp (coef, every) or None
+    multiplies the queries of position p by 1 + coef ln(floor((p + 1) / every) + 1)."""
+    T, H, D = q.shape
+    G = k.shape[1]
+    pos = torch.arange(T)
+    if q_temp:
+        temp = 1.0 + q_temp[0] * torch.log(torch.floor((pos + 1).to(F64) / q_temp[1]) + 1.0)
+        q = q * temp[:, None, None]
+    dist = pos[:, None] - pos[None, :]
+    seen = (dist >= 0) & ((dist < window) if window is not None else True)
+    out = torch.zeros(T, H, v.shape[2], dtype=F64)
+    for hh in range(H):
+        g = hh // (H // G)
+        slope = 2.0 ** (-8.0 * (hh + 1) / H)
+        s = (q[:, hh] @ k[:, g].T) * scale - slope * dist.to(F64)
+        s = s.masked_fill(~seen, -math.inf)
+        out[:, hh] = torch.softmax(s, -1) @ v[:, g]
+    return out
+
+
 def window_attention(h, m, w, p, eps):
     T = h.shape[0]
     H, G, D = m["heads"], m["kv_heads"], m["dim"]
     q = (h @ w[p + "q"].T).view(T, H, D)
     kraw = (h @ w[p + "k"].T).view(T, G, D)
-    v = kraw                                                    # the values are the keys as projected
     q = rms_norm(q, w[p + "q.norm"], eps)
     k = rms_norm(kraw, w[p + "k.norm"], eps)
-    pos = torch.arange(T)
     qt = m.get("q_temp")
-    if qt:
-        temp = 1.0 + qt["coef"] * torch.log(torch.floor((pos + 1).to(F64) / qt["every"]) + 1.0)
-        q = q * temp[:, None, None]
-    dist = pos[:, None] - pos[None, :]
     size = m["mask"]["size"] if m.get("mask") else None
-    seen = (dist >= 0) & ((dist < size) if size is not None else True)
-    out = torch.zeros(T, H, D, dtype=F64)
-    for hh in range(H):
-        g = hh // (H // G)
-        slope = 2.0 ** (-8.0 * (hh + 1) / H)
-        s = (q[:, hh] @ k[:, g].T) * m["scale"] - slope * dist.to(F64)
-        s = s.masked_fill(~seen, -math.inf)
-        out[:, hh] = torch.softmax(s, -1) @ v[:, g]
+    # the values are the keys as projected, before their norm
+    out = sloped_window_softmax(q, k, kraw, m["scale"], size, (qt["coef"], qt["every"]) if qt else None)
     return out.reshape(T, H * D) @ w[p + "o"].T
 
 
@@ -205,6 +215,16 @@ def rotate_pairs(x, base, dims):
     return y
 
 
+def causal_sink_softmax(s, sink):
+    """Softmax weights of the scores s [T, T] over j <= i; the denominator also holds exp(sink), which
+    has no key and no value, is not scaled and counts once."""
+    T = s.shape[0]
+    pos = torch.arange(T)
+    s = s.masked_fill(pos[:, None] < pos[None, :], -math.inf)
+    s = torch.cat([s, sink.expand(T, 1)], 1)
+    return torch.softmax(s, -1)[:, :T]
+
+
 def latent_attention(h, m, w, p, eps):
     T = h.shape[0]
     H, D, rd, Dv, R = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
@@ -215,15 +235,10 @@ def latent_attention(h, m, w, p, eps):
     k_rot = rotate_pairs(z[:, R:], m["rot"]["base"], m["rot"]["dims"])     # one rotated key part for all heads
     k_plain = (c @ w[p + "uk"].T).view(T, H, D)
     v = (c @ w[p + "uv"].T).view(T, H, Dv)
-    pos = torch.arange(T)
-    seen = pos[:, None] >= pos[None, :]
     out = torch.zeros(T, H, Dv, dtype=F64)
     for hh in range(H):
         s = (q_plain[:, hh] @ k_plain[:, hh].T + q_rot[:, hh] @ k_rot.T) * m["scale"]
-        s = s.masked_fill(~seen, -math.inf)
-        # the sink joins the denominator once, with no value
-        s = torch.cat([s, w[p + "sink"][hh].expand(T, 1)], 1)
-        out[:, hh] = torch.softmax(s, -1)[:, :T] @ v[:, hh]
+        out[:, hh] = causal_sink_softmax(s, w[p + "sink"][hh]) @ v[:, hh]
     return out.reshape(T, H * Dv) @ w[p + "o"].T
 
 
@@ -278,3 +293,10 @@ def forward(cfg, weights, tokens, layers_out=None, choice=None):
         if layers_out is not None:
             layers_out.append(x)
     return layer_norm(x, w["final.norm"], w["final.norm.b"], eps) @ w["head"].T
+
+
+def greedy(cfg, weights, prompt, n):
+    toks = list(prompt)
+    for _ in range(n):
+        toks.append(int(forward(cfg, weights, toks)[-1].argmax()))
+    return toks[len(prompt):]
