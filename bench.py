@@ -92,11 +92,14 @@ def build_parser() -> argparse.ArgumentParser:
                     help="single-stage layouts: host waits for each step's tokens before scheduling the "
                          "next (default: EngineConfig.async_decode, the next step overlaps the host work)")
     ap.add_argument("--out", default=None, help="also write the JSON line here")
-    ap.add_argument("--mixer-family", default="nesizen", choices=["nesizen", "zinesun", "lizizen"],
+    ap.add_argument("--mixer-family", default="nesizen", choices=["nesizen", "zinesun", "lizizen", "gevipel"],
                     help="with --mixer-compare: the heterogeneous family that is timed (nesizen: beside a Mixtral "
                          "stack; zinesun: latent attention beside a Nesizen stack of plain windowed attention; "
                          "lizizen: parallel layers of distance-biased and differential attention with dense GLU "
-                         "feed-forwards beside a Nesizen stack of plain attention with dense feed-forwards)")
+                         "feed-forwards beside a Nesizen stack of plain attention with dense feed-forwards; "
+                         "gevipel: sandwich-normed layers of sloped window attention, the gated delta rule and latent "
+                         "attention with a sink over routed plain experts beside a Nesizen stack of windowed "
+                         "attention and gated linear attention over routed GLU experts)")
     ap.add_argument("--mixer-compare", default=None, metavar="SIZES",
                     help="instead of the headline run: prefill and decode throughput of a Nesizen stack "
                          "(windowed attention, shared keys, gated linear attention, sigmoid MoE) beside a "
@@ -223,6 +226,31 @@ def run_mixer_compare(a) -> int:
                                                   "mlp": dns} for w in (1 << 30, win, 1 << 30, win)]},
                                             name=f"nesizen-dense-{size}")
             pair = (liz, nes3)
+        if a.mixer_family == "gevipel":
+            # sloped window attention (values = keys), the gated delta rule with 4-tap convolutions, causal
+            # latent attention with a sink (cached rows 192 + 64 wide), all over routed squared-ReLU experts
+            # of 3/2 the width (two matrices: the parameters and FLOPs of a GLU expert's three), beside windowed
+            # GQA attention and gated linear attention of the same heads over routed GLU experts, one stream
+            slo = {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5, "mask": {"size": win},
+                   "q_temp": {"coef": 0.1, "every": 128}}
+            dlt = {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "conv": 4}
+            lat = {"heads": H, "dim": D, "rot_dim": 64, "vdim": D, "kv_rank": 192, "rot": {"dims": 64, "base": 1e6},
+                   "scale": (D + 64) ** -0.5}
+            pmoe = {"kind": "moe", "expert": {"ff": 3 * eff // 2}, "router": {"experts": E, "top": top}}
+            gev = ModelConfig.from_gevipel({"architecture": "Gevipel", "vocab": 32000, "width": W, "norm": {"eps": 1e-6},
+                                            "embedding": {"scale": W ** 0.5}, "residual_mult": 0.5, "layers": [
+                                                {"type": t, "mixer": m, "mlp": pmoe} for t, m in
+                                                (("attention", slo), ("delta", dlt), ("latent_attention", lat),
+                                                 ("delta", dlt))]}, name=f"gevipel-{size}")
+            plain = dict(attn, mask={"size": win, "keep_first": 0})
+            nes4 = ModelConfig.from_nesizen({"architecture": "Nesizen", "vocab": 32000, "width": W, "streams": 1,
+                                             "norm": {"eps": 1e-6}, "layers": [
+                                                 {"type": "attention", "mixer": plain, "mlp": moe},
+                                                 {"type": "gla", "mixer": gla, "mlp": moe},
+                                                 {"type": "attention", "mixer": dict(plain, mask={"size": 1 << 30, "keep_first": 0}),
+                                                  "mlp": moe},
+                                                 {"type": "gla", "mixer": gla, "mlp": moe}]}, name=f"nesizen-mix-{size}")
+            pair = (gev, nes4)
         for cfg in pair:
             ecfg = EngineConfig(max_batch=B, max_seq_len=P + K + Wm + 8, max_prefill_tokens=8192,
                                 kv_cache_tokens=B * (P + K + Wm + 40), use_graphs=not a.no_graphs,
