@@ -42,8 +42,9 @@ __device__ __forceinline__ void row_stats(const float* __restrict__ sy, int W, f
   rstd = 1.f / sqrtf(block_sum(q, red) / (float)W + eps);
 }
 
-// One workgroup per row; the row of y, then the updated row of x, staged in LDS.
-template <typename T>
+// One workgroup per row; the row of y, then the updated row of x, staged in LDS. V = 4 (W % 4 == 0):
+// 16-byte accesses (8-byte for bf16); the statistics are the same two-pass sums either way.
+template <typename T, int V>
 __global__ __launch_bounds__(1024) void post_norm_add_norm_kernel(float* __restrict__ x, const T* __restrict__ y,
                                                                  const float* __restrict__ nw,
                                                                  const float* __restrict__ nb, float eps, float mult,
@@ -51,23 +52,46 @@ __global__ __launch_bounds__(1024) void post_norm_add_norm_kernel(float* __restr
                                                                  const float* __restrict__ nw2,
                                                                  const float* __restrict__ nb2, T* __restrict__ h,
                                                                  int W) {
-  extern __shared__ float sy[];
+  typedef float fv __attribute__((ext_vector_type(V)));
+  typedef T tv __attribute__((ext_vector_type(V)));
+  extern __shared__ __attribute__((aligned(16))) float sy[];
   __shared__ float red[16];
   const long t = blockIdx.x;
-  for (int c = threadIdx.x; c < W; c += blockDim.x) sy[c] = (float)y[t * W + c];
+  for (int c = V * threadIdx.x; c < W; c += V * blockDim.x) {
+    const tv yv = *reinterpret_cast<const tv*>(y + t * W + c);
+    fv f;
+#pragma unroll
+    for (int e = 0; e < V; ++e) f[e] = (float)yv[e];
+    *reinterpret_cast<fv*>(sy + c) = f;
+  }
   __syncthreads();
   float mean, rstd;
   row_stats(sy, W, eps, red, mean, rstd);
-  for (int c = threadIdx.x; c < W; c += blockDim.x) {
-    float v = x[t * W + c] + mult * ((sy[c] - mean) * rstd * nw[c] + nb[c]);
-    if (extra) v += extra[t * W + c];
-    x[t * W + c] = v;
-    sy[c] = v;              // (this thread's own elements: no other thread reads them before the barrier)
+  for (int c = V * threadIdx.x; c < W; c += V * blockDim.x) {
+    const fv yv = *reinterpret_cast<const fv*>(sy + c), wv = *reinterpret_cast<const fv*>(nw + c),
+             bv = *reinterpret_cast<const fv*>(nb + c);
+    fv v = *reinterpret_cast<const fv*>(x + t * W + c);
+#pragma unroll
+    for (int e = 0; e < V; ++e) v[e] = v[e] + mult * ((yv[e] - mean) * rstd * wv[e] + bv[e]);
+    if (extra) {
+      const fv ev = *reinterpret_cast<const fv*>(extra + t * W + c);
+#pragma unroll
+      for (int e = 0; e < V; ++e) v[e] += ev[e];
+    }
+    *reinterpret_cast<fv*>(x + t * W + c) = v;
+    *reinterpret_cast<fv*>(sy + c) = v;      // (a thread rewrites only what it alone read after the barrier)
   }
   if (!h) return;
   __syncthreads();
   row_stats(sy, W, eps, red, mean, rstd);
-  for (int c = threadIdx.x; c < W; c += blockDim.x) h[t * W + c] = (T)((sy[c] - mean) * rstd * nw2[c] + nb2[c]);
+  for (int c = V * threadIdx.x; c < W; c += V * blockDim.x) {
+    const fv xv = *reinterpret_cast<const fv*>(sy + c), wv = *reinterpret_cast<const fv*>(nw2 + c),
+             bv = *reinterpret_cast<const fv*>(nb2 + c);
+    tv o;
+#pragma unroll
+    for (int e = 0; e < V; ++e) o[e] = (T)((xv[e] - mean) * rstd * wv[e] + bv[e]);
+    *reinterpret_cast<tv*>(h + t * W + c) = o;
+  }
 }
 
 // one thread per (row, channel); the taps are summed oldest first
@@ -100,6 +124,86 @@ __global__ __launch_bounds__(256) void short_conv_act_kernel(const TI* __restric
   out[(long)t * C + c] = (TO)acc;
 }
 
+// The same for up to 8 taps and C % 4 == 0 with RB consecutive rows per workgroup: a thread owns 4
+// channels, keeps their last taps - 1 inputs in registers and slides over the rows, so a row costs one
+// load of z; the history is fetched anew (earlier rows, the pool, or zeros) at the block's first row and
+// wherever a new sequence begins. Taps are summed in the same order as above.
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void short_conv_act_rows_kernel(const TI* __restrict__ z, long z_ld,
+                                                                  const float* __restrict__ w,
+                                                                  const float* __restrict__ state,
+                                                                  const int* __restrict__ state_slots,
+                                                                  const int* __restrict__ row_cu, int nseq,
+                                                                  const int* __restrict__ positions,
+                                                                  TO* __restrict__ out, int C, int taps, int act, int T,
+                                                                  int RB) {
+  constexpr int MAXN = 7;
+  typedef TI tiv __attribute__((ext_vector_type(4)));
+  typedef TO tov __attribute__((ext_vector_type(4)));
+  const int t0 = blockIdx.x * RB, t1 = min(T, t0 + RB);
+  const int c = (blockIdx.y * blockDim.x + threadIdx.x) * 4;
+  if (c >= C) return;
+  const int n = taps - 1;
+  f32x4 wv[MAXN + 1], hist[MAXN];
+#pragma unroll
+  for (int j = 0; j <= MAXN; ++j)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) wv[j][e] = j < taps ? w[(long)(c + e) * taps + j] : 0.f;
+  auto ld = [&](long row) {
+    const tiv v = *reinterpret_cast<const tiv*>(z + row * z_ld + c);
+    return f32x4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+  };
+  int s = -1, send = t0;
+  bool fetch = true;
+  for (int t = t0; t < t1; ++t) {
+    if (t >= send) {
+      s = seq_of_row(row_cu, nseq, t);
+      send = s >= 0 ? row_cu[s + 1] : t + 1;
+      fetch = true;
+    }
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    if (s >= 0) {
+      const f32x4 zc = ld(t);
+      if (fetch) {
+        const int a = row_cu[s], p = positions[t];
+        const int slot = state_slots ? state_slots[s] : -1;
+#pragma unroll
+        for (int k = 0; k < MAXN; ++k) {
+          if (k >= n) break;
+          const int d = n - k;
+          f32x4 v = {0.f, 0.f, 0.f, 0.f};
+          if (t - d >= a) v = ld(t - d);
+          else if (p - d >= 0 && slot >= 0)
+            v = *reinterpret_cast<const f32x4*>(state + ((long)slot * n + (n - (d - (t - a)))) * C + c);
+          hist[k] = v;
+        }
+        fetch = false;
+      }
+#pragma unroll
+      for (int k = 0; k < MAXN; ++k) {
+        if (k >= n) break;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] = fmaf(wv[k][e], hist[k][e], acc[e]);
+      }
+#pragma unroll
+      for (int k = 0; k <= MAXN; ++k)
+        if (k == n) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[e] = fmaf(wv[k][e], zc[e], acc[e]);
+        }
+#pragma unroll
+      for (int k = 0; k < MAXN; ++k) {
+        if (k + 1 < n) hist[k] = hist[k + 1];
+        else if (k + 1 == n) hist[k] = zc;
+      }
+    }
+    tov o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = (TO)(act == 1 ? acc[e] / (1.f + expf(-acc[e])) : acc[e]);
+    *reinterpret_cast<tov*>(out + (long)t * C + c) = o;
+  }
+}
+
 // one thread per (sequence, channel): entry i of the new history is old entry i + len while that
 // exists (read before any entry at or above it is written), then the step's own rows
 template <typename TI>
@@ -123,14 +227,27 @@ __global__ __launch_bounds__(256) void short_conv_state_update_kernel(const TI* 
   }
 }
 
+// sum over the 8 lanes that share lane >> 3, in every lane, by three cross-lane moves inside a row of 16
+// (neighbour, next pair, mirrored half row): no LDS traffic, so the token loop's LDS reads stay in flight
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float sum8(float v) {
+  v += dpp_move<0xB1>(v);      // quad_perm [1, 0, 3, 2]
+  v += dpp_move<0x4E>(v);      // quad_perm [2, 3, 0, 1]
+  v += dpp_move<0x141>(v);     // row_half_mirror: lane i of 8 <- lane 7 - i (the other quad's sum)
+  return v;
+}
+
 // Workgroup = (sequence, head, 64-column slice of Dv), 8 waves; wave w owns 8 columns. A lane is
-// (column c = lane & 7, row group gg = lane >> 3) and keeps the NR rows d = gg * NR .. + NR - 1 of its
+// (row group gg = lane & 7, column c = lane >> 3) and keeps the NR rows d = gg * NR .. + NR - 1 of its
 // column's state in registers. Tokens are staged 16 at a time: raw keys and queries go to LDS (rows
 // past D are zero, so the row loop needs no bound), and per token the five scalars of the update:
 // decay g, write strength beta, 1 / |k|, q_scale / |q| (the unit norms are folded into scalars:
 // S^T k = kn S^T k_raw and so on, so no element is normalised on its own). A token then costs a dot
-// product of the lane's rows with k, three shuffles to sum the eight row groups, one fused pass that
-// updates the rows and accumulates the read-out, and three more shuffles: no barrier inside the token
+// product of the lane's rows with k, three cross-lane moves to sum the eight row groups, one fused pass that
+// updates the rows and accumulates the read-out, and three more moves: no barrier inside the token
 // loop. The outputs of the 16 tokens leave through LDS.
 template <typename T, int NR>
 __global__ __launch_bounds__(512) void delta_scan_kernel(const float* __restrict__ q, long q_ld,
@@ -151,7 +268,7 @@ __global__ __launch_bounds__(512) void delta_scan_kernel(const float* __restrict
   const int s = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * 64;
   const int hk = h / (H / G);
   const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int cl = 8 * w + (lane & 7), gg = lane >> 3;
+  const int cl = 8 * w + (lane >> 3), gg = lane & 7;
   const int col = c0 + cl;
   const bool live = col < Dv;
   const int r0 = row_cu[s], r1 = row_cu[s + 1];
@@ -218,9 +335,7 @@ __global__ __launch_bounds__(512) void delta_scan_kernel(const float* __restrict
 #pragma unroll
         for (int j = 0; j < 4; ++j) dot = fmaf(st[4 * i4 + j], kr[i4][j], dot);
       }
-      dot += __shfl_xor(dot, 8, 64);
-      dot += __shfl_xor(dot, 16, 64);
-      dot += __shfl_xor(dot, 32, 64);
+      dot = sum8(dot);
       // the decayed state's read at k is g kn dot; the write is k_unit u^T = k_raw (kn u)
       const float u = bt * (vv - g * (kn * dot));
       const float uk = kn * u;
@@ -234,9 +349,7 @@ __global__ __launch_bounds__(512) void delta_scan_kernel(const float* __restrict
           po = fmaf(q4[j], st[4 * i4 + j], po);
         }
       }
-      po += __shfl_xor(po, 8, 64);
-      po += __shfl_xor(po, 16, 64);
-      po += __shfl_xor(po, 32, 64);
+      po = sum8(po);
       if (gg == 0) so[tt][cl] = po * qn;
     }
     __syncthreads();
@@ -266,18 +379,32 @@ void launch_post_norm_add_norm(float* x, const void* y, const float* nw, const f
                                hipStream_t s) {
   if (T <= 0) return;
   const size_t sm = (size_t)W * sizeof(float);
-  if (f32)
-    post_norm_add_norm_kernel<float><<<T, row_threads(W), sm, s>>>(x, (const float*)y, nw, nb, eps, mult, extra, nw2, nb2,
-                                                                  (float*)h, W);
-  else
-    post_norm_add_norm_kernel<bf16><<<T, row_threads(W), sm, s>>>(x, (const bf16*)y, nw, nb, eps, mult, extra, nw2, nb2,
-                                                                 (bf16*)h, W);
+#define BFLY_PNAN(TT, V)                                                                                          \
+  post_norm_add_norm_kernel<TT, V><<<T, row_threads(W), sm, s>>>(x, (const TT*)y, nw, nb, eps, mult, extra, nw2, nb2, \
+                                                                 (TT*)h, W)
+  if (W % 4 == 0) { if (f32) BFLY_PNAN(float, 4); else BFLY_PNAN(bf16, 4); }
+  else { if (f32) BFLY_PNAN(float, 1); else BFLY_PNAN(bf16, 1); }
+#undef BFLY_PNAN
 }
 
 void launch_short_conv_act(const void* z, long z_ld, const float* w, const float* state, const int* state_slots,
                            const int* row_cu, int nseq, const int* positions, void* out, int T, int C, int taps, int act,
                            bool f32, bool out_f32, hipStream_t s) {
   if (T <= 0 || C <= 0) return;
+  const size_t esz = f32 ? 4 : 2;
+  if (taps <= 8 && C % 4 == 0 && z_ld % 4 == 0 && reinterpret_cast<uintptr_t>(z) % (4 * esz) == 0 && T >= 64) {
+    // rows per workgroup: enough workgroups to fill the chip first
+    const int RB = std::min(16, std::max(1, T / 512));
+    dim3 g2((T + RB - 1) / RB, (C / 4 + 255) / 256);
+#define BFLY_SCR(TI, TO)                                                                                             \
+  short_conv_act_rows_kernel<TI, TO><<<g2, 256, 0, s>>>((const TI*)z, z_ld, w, state, state_slots, row_cu, nseq,     \
+                                                        positions, (TO*)out, C, taps, act, T, RB)
+    if (f32) BFLY_SCR(float, float);
+    else if (out_f32) BFLY_SCR(bf16, float);
+    else BFLY_SCR(bf16, bf16);
+#undef BFLY_SCR
+    return;
+  }
   dim3 grid(T, (C + 255) / 256);
 #define BFLY_SC(TI, TO)                                                                                              \
   short_conv_act_kernel<TI, TO><<<grid, 256, 0, s>>>((const TI*)z, z_ld, w, state, state_slots, row_cu, nseq, positions, \

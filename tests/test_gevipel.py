@@ -158,6 +158,35 @@ def test_short_convolution_through_packed_steps(target, taps, C):
     assert y.dtype == dt and close(y, O.short_conv(z[0][:5], w), dt)
 
 
+@pytest.mark.parametrize("taps,C", [(4, 256), (8, 72), (9, 64), (3, 130)])
+def test_short_convolution_in_large_steps(target, taps, C):
+    """Steps of hundreds of rows (a thread slides over rows with the history in registers): two prompts
+    and a decoded row in one step, then their continuations from the history pool; bf16 output."""
+    dev, dt = target
+    lens = [260, 150, 40]
+    z = [rnd(n, C, seed=20 + s) for s, n in enumerate(lens)]
+    w = rnd(C, taps, seed=4, scale=0.5)
+    want = [O.silu(O.short_conv(z[s], w)) for s in range(3)]
+    state = torch.full((3, taps - 1, C), -3.0, dtype=torch.float32, device=dev)
+    at, got = [0, 0, 0], [[] for _ in lens]
+    for step in ([(2, 39)], [(2, 1), (0, 200), (1, 97)], [(0, 60), (1, 53)]):
+        cu, pos = packed_step([(at[s], c) for s, c in step], dev)
+        zin = torch.cat([z[s][at[s]:at[s] + c] for s, c in step]).to(dt).to(dev)
+        sl = i32([s for s, _ in step], dev)
+        y = ops.short_conv_act(zin, w.float().to(dev), state, sl, cu, pos, "silu", torch.float32)
+        y2 = ops.short_conv_act(zin, w.float().to(dev), state, sl, cu, pos, "silu", dt)
+        assert close(y2, y.double().cpu(), dt)
+        ops.short_conv_state_update_(zin, state, sl, cu, pos)
+        r = 0
+        for s, c in step:
+            got[s].append(y[r:r + c])
+            r += c
+            at[s] += c
+    assert at == lens
+    for s in range(3):
+        assert close(torch.cat(got[s]), want[s], dt), f"sequence {s}"
+
+
 def delta_inputs(T, H, G, D, Dv, seed):
     q, k, v = rnd(T, G, D, seed=seed), rnd(T, G, D, seed=seed + 1), rnd(T, H, Dv, seed=seed + 2)
     b, a = rnd(T, H, seed=seed + 3, scale=2.0), rnd(T, H, seed=seed + 4, scale=2.0)
