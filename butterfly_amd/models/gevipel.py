@@ -301,13 +301,13 @@ class GevipelLM(PackedStack):
 
     def allocate_state(self, num_slots: int) -> list:
         """Two f32 tensors per run of a delta layer: the last taps - 1 projected q | k | v rows
-        [slots, taps - 1, C] (oldest first) and the delta-rule matrices [slots, H, D, Dv]."""
+        [slots, taps - 1, C] (oldest first) and the delta-rule matrices, column by column [slots, H, Dv, D]."""
         self.state = []
         for r in sorted(self.state_index, key=self.state_index.get):
             sp = self.specs[self.runs[r]]
             self.state.append(torch.zeros(num_slots, sp["taps"] - 1, self._conv_channels(sp), dtype=torch.float32,
                                           device=self.device))
-            self.state.append(torch.zeros(num_slots, sp["heads"], sp["dim"], sp["vdim"], dtype=torch.float32,
+            self.state.append(torch.zeros(num_slots, sp["heads"], sp["vdim"], sp["dim"], dtype=torch.float32,
                                           device=self.device))
         return self.state
 

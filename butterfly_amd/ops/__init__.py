@@ -1231,8 +1231,8 @@ def short_conv_state_update_(z, state, state_slots, row_cu, positions):
 
 def delta_scan(q, k, v, b, a, a_log, dt_bias, state, state_slots, row_cu, positions, q_scale: float,
                unit_eps: float = 1e-6):
-    """Gated delta rule over packed rows with the state pooled in `state` [slots, H, D, Dv] f32
-    (updated in place; a sequence whose step starts at position 0 starts from zero). q, k [T, G, D],
+    """Gated delta rule over packed rows with the state pooled in `state` [slots, H, Dv, D] f32 (a
+    head's D x Dv matrix stored column by column; updated in place; a sequence whose step starts at position 0 starts from zero). q, k [T, G, D],
     v [T, H, Dv] (views allowed); b, a [T, H] the logits of the write strength and the decay's step;
     a_log, dt_bias [H] f32. See ops.reference.delta_scan. Returns o [T, H, Dv] f32."""
     if not _gpu(q):

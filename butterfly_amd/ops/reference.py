@@ -1056,8 +1056,9 @@ def delta_scan(q, k, v, b, a, a_log, dt_bias, state, state_slots, row_cu, positi
     query / key group h // (H / G)); q and k are first made unit vectors, x / sqrt(sum x^2 +
     unit_eps), and q is multiplied by q_scale. Per row and head: beta = sigmoid(b), decay =
     exp(-exp(a_log[h]) softplus(a + dt_bias[h])); S <- decay S; u = beta (v - S^T k); S <- S + k u^T;
-    o = S^T q. The state S [D, Dv] of sequence s is read from state[state_slots[s]] unless its first
-    row is at position 0 (then zero) and written back after its last row. Returns o [T, H, Dv] f32."""
+    o = S^T q. The state S [D, Dv] of sequence s is read from state[state_slots[s]] (stored column by
+    column, [H, Dv, D]) unless its first row is at position 0 (then zero) and written back after its
+    last row. Returns o [T, H, Dv] f32."""
     T, G, D = q.shape
     H, Dv = v.shape[1], v.shape[2]
     rep = H // G
@@ -1072,11 +1073,12 @@ def delta_scan(q, k, v, b, a, a_log, dt_bias, state, state_slots, row_cu, positi
     for s in range(len(cu) - 1):
         if cu[s + 1] == cu[s] or sl[s] < 0:
             continue
-        S = torch.zeros(H, D, Dv, dtype=torch.float32, device=q.device) if pos[cu[s]] == 0 else state[sl[s]].clone()
+        S = torch.zeros(H, D, Dv, dtype=torch.float32, device=q.device) if pos[cu[s]] == 0 \
+            else state[sl[s]].transpose(1, 2).clone()
         for t in range(cu[s], cu[s + 1]):
             S = decay[t][:, None, None] * S
             u = beta[t][:, None] * (vf[t] - torch.einsum("hdv,hd->hv", S, kf[t]))
             S = S + kf[t][:, :, None] * u[:, None, :]
             o[t] = torch.einsum("hdv,hd->hv", S, qf[t])
-        state[sl[s]] = S
+        state[sl[s]] = S.transpose(1, 2)
     return o

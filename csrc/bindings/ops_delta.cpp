@@ -113,7 +113,8 @@ void delta_scan(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor&
   TORCH_CHECK(b.dim() == 2 && a.dim() == 2 && b.stride(1) == 1 && a.stride(1) == 1 && b.size(0) == T && a.size(0) == T &&
                   b.size(1) == H && a.size(1) == H && a_log.numel() == H && dt_bias.numel() == H,
               "delta_scan: b / a [T, H], a_log / dt_bias [H]");
-  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == D && state.size(3) == Dv, "delta_scan: state");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == Dv && state.size(3) == D,
+              "delta_scan: state [slots, H, Dv, D]");
   check_step(state_slots, row_cu, positions, T, state.size(0), "delta_scan");
   TORCH_CHECK(o.dim() == 3 && o.size(0) == T && o.size(1) == H && o.size(2) == Dv, "delta_scan: o");
   const int rc = bfly::launch_delta_scan(q.data_ptr<float>(), q.stride(0), k.data_ptr<float>(), k.stride(0),

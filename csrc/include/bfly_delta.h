@@ -24,7 +24,8 @@ void launch_short_conv_act(const void* z, long z_ld, const float* w, const float
 void launch_short_conv_state_update(const void* z, long z_ld, float* state, const int* state_slots, const int* row_cu,
                                     int nseq, const int* positions, int C, int n, bool f32, hipStream_t s);
 // Gated delta rule over packed rows (see ops.delta_scan): q, k f32 [T, G, D], v f32 [T, H, Dv] with row
-// strides, b / a [T, H] logits of the activation type, state f32 [slots, H, D, Dv], o f32 [T, H, Dv].
+// strides, b / a [T, H] logits of the activation type, state f32 [slots, H, Dv, D] (a head's state
+// column by column), o f32 [T, H, Dv].
 // Returns < 0 if D > 256.
 int launch_delta_scan(const float* q, long q_ld, const float* k, long k_ld, const float* v, long v_ld, const void* b,
                       long b_ld, const void* a, long a_ld, const float* a_log, const float* dt_bias, float* state,

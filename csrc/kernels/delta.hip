@@ -242,13 +242,15 @@ __device__ __forceinline__ float sum8(float v) {
 
 // Workgroup = (sequence, head, 64-column slice of Dv), 8 waves; wave w owns 8 columns. A lane is
 // (row group gg = lane & 7, column c = lane >> 3) and keeps the NR rows d = gg * NR .. + NR - 1 of its
-// column's state in registers. Tokens are staged 16 at a time: raw keys and queries go to LDS (rows
-// past D are zero, so the row loop needs no bound), and per token the five scalars of the update:
-// decay g, write strength beta, 1 / |k|, q_scale / |q| (the unit norms are folded into scalars:
-// S^T k = kn S^T k_raw and so on, so no element is normalised on its own). A token then costs a dot
-// product of the lane's rows with k, three cross-lane moves to sum the eight row groups, one fused pass that
-// updates the rows and accumulates the read-out, and three more moves: no barrier inside the token
-// loop. The outputs of the 16 tokens leave through LDS.
+// column's state in registers. The pool holds a head's state column by column ([Dv, D]: the rows a lane
+// owns are contiguous, the eight lanes of a column cover it with 16-byte accesses). Tokens are staged
+// 16 at a time: raw keys and queries go to LDS (rows past D are zero, so the row loop needs no bound),
+// and per token the scalars of the update: decay g, write strength beta, 1 / |k|, q_scale / |q| (the
+// unit norms are folded into scalars: S^T k = kn S^T k_raw and so on, so no element is normalised on
+// its own). The next block's inputs travel to registers while the current block is computed. A token
+// then costs a dot product of the lane's rows with k (four partial sums), three cross-lane moves to sum
+// the eight row groups, one fused pass that updates the rows and accumulates the read-out, and three
+// more moves: no barrier inside the token loop. The outputs of the 16 tokens leave through LDS.
 template <typename T, int NR>
 __global__ __launch_bounds__(512) void delta_scan_kernel(const float* __restrict__ q, long q_ld,
                                                          const float* __restrict__ k, long k_ld,
@@ -261,7 +263,7 @@ __global__ __launch_bounds__(512) void delta_scan_kernel(const float* __restrict
                                                          const int* __restrict__ positions, float q_scale,
                                                          float unit_eps, float* __restrict__ o, int H, int G, int D,
                                                          int Dv) {
-  constexpr int TB = 16, DP = 8 * NR, NT = 512;
+  constexpr int TB = 16, DP = 8 * NR, NT = 512, KQ = TB * DP / NT, VN = TB * 64 / NT;
   __shared__ __attribute__((aligned(16))) float sk[TB * DP], sq[TB * DP];
   __shared__ float sv[TB][64], so[TB][64];
   __shared__ float sg[TB], sb[TB], skn[TB], sqn[TB];
@@ -279,33 +281,61 @@ __global__ __launch_bounds__(512) void delta_scan_kernel(const float* __restrict
       if (c0 + (i & 63) < Dv) o[((long)(r0 + (i >> 6)) * H + h) * Dv + c0 + (i & 63)] = 0.f;
     return;
   }
-  float* S = state + ((long)slot * H + h) * D * Dv;
+  float* S = state + (((long)slot * H + h) * Dv + col) * D;      // this lane's column
+  const bool vec = (D & 3) == 0;
   float st[NR];
   const bool fresh = positions[r0] == 0;
 #pragma unroll
-  for (int i = 0; i < NR; ++i) {
-    const int d = gg * NR + i;
-    st[i] = (!fresh && live && d < D) ? S[(long)d * Dv + col] : 0.f;
+  for (int i4 = 0; i4 < NR / 4; ++i4) {
+    const int d = gg * NR + 4 * i4;
+    f32x4 x = {0.f, 0.f, 0.f, 0.f};
+    if (!fresh && live) {
+      if (vec && d + 3 < D) x = *reinterpret_cast<const f32x4*>(S + d);
+      else
+#pragma unroll
+        for (int j = 0; j < 4; ++j) x[j] = d + j < D ? S[d + j] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) st[4 * i4 + j] = x[j];
   }
   const float rate = expf(a_log[h]), dtb = dt_bias[h];
-  for (int t0 = r0; t0 < r1; t0 += TB) {
+  // the inputs of a block of TB tokens, one slice per thread
+  float rk[KQ], rq[KQ], rv[VN], ra = 0.f, rb = 0.f;
+  auto fetch = [&](int t0) {
     const int nb = min(TB, r1 - t0);
-    for (int i = threadIdx.x; i < nb * DP; i += NT) {
-      const int tt = i / DP, d = i - tt * DP;
+#pragma unroll
+    for (int j = 0; j < KQ; ++j) {
+      const int i = threadIdx.x + j * NT, tt = i / DP, d = i - tt * DP;
+      const bool ok = tt < nb && d < D;
       const long t = t0 + tt;
-      sk[i] = d < D ? k[t * k_ld + (long)hk * D + d] : 0.f;
-      sq[i] = d < D ? q[t * q_ld + (long)hk * D + d] : 0.f;
+      rk[j] = ok ? k[t * k_ld + (long)hk * D + d] : 0.f;
+      rq[j] = ok ? q[t * q_ld + (long)hk * D + d] : 0.f;
     }
-    for (int i = threadIdx.x; i < nb * 64; i += NT) {
-      const int tt = i >> 6, c = i & 63;
-      sv[tt][c] = (c0 + c < Dv) ? v[(long)(t0 + tt) * v_ld + (long)h * Dv + c0 + c] : 0.f;
+#pragma unroll
+    for (int j = 0; j < VN; ++j) {
+      const int i = threadIdx.x + j * NT, tt = i >> 6, c = i & 63;
+      rv[j] = (tt < nb && c0 + c < Dv) ? v[(long)(t0 + tt) * v_ld + (long)h * Dv + c0 + c] : 0.f;
     }
     if (threadIdx.x < nb) {
-      const long t = t0 + threadIdx.x;
-      const float av = (float)al[t * a_ld + h] + dtb;
+      ra = (float)al[(long)(t0 + threadIdx.x) * a_ld + h];
+      rb = (float)bl[(long)(t0 + threadIdx.x) * b_ld + h];
+    }
+  };
+  fetch(r0);
+  for (int t0 = r0; t0 < r1; t0 += TB) {
+    const int nb = min(TB, r1 - t0);
+#pragma unroll
+    for (int j = 0; j < KQ; ++j) {
+      sk[threadIdx.x + j * NT] = rk[j];
+      sq[threadIdx.x + j * NT] = rq[j];
+    }
+#pragma unroll
+    for (int j = 0; j < VN; ++j) sv[(threadIdx.x + j * NT) >> 6][threadIdx.x & 63] = rv[j];
+    if (threadIdx.x < nb) {
+      const float av = ra + dtb;
       const float sp = av > 20.f ? av : log1pf(expf(av));            // softplus
       sg[threadIdx.x] = expf(-rate * sp);
-      sb[threadIdx.x] = 1.f / (1.f + expf(-(float)bl[t * b_ld + h]));
+      sb[threadIdx.x] = 1.f / (1.f + expf(-rb));
     }
     __syncthreads();
     // unit norms: wave w sums the squares of tokens w and w + 8
@@ -323,33 +353,34 @@ __global__ __launch_bounds__(512) void delta_scan_kernel(const float* __restrict
       }
     }
     __syncthreads();
+    if (t0 + TB < r1) fetch(t0 + TB);        // in flight during the token loop
     for (int tt = 0; tt < nb; ++tt) {
       const float vv = sv[tt][cl], g = sg[tt], bt = sb[tt], kn = skn[tt], qn = sqn[tt];
       const f32x4* pk = reinterpret_cast<const f32x4*>(sk + tt * DP + gg * NR);
       const f32x4* pq = reinterpret_cast<const f32x4*>(sq + tt * DP + gg * NR);
       f32x4 kr[NR / 4];
-      float dot = 0.f;
+      f32x4 dp = {0.f, 0.f, 0.f, 0.f};      // four partial sums: short dependent chains
 #pragma unroll
       for (int i4 = 0; i4 < NR / 4; ++i4) {
         kr[i4] = pk[i4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) dot = fmaf(st[4 * i4 + j], kr[i4][j], dot);
+        for (int j = 0; j < 4; ++j) dp[j] = fmaf(st[4 * i4 + j], kr[i4][j], dp[j]);
       }
-      dot = sum8(dot);
+      const float dot = sum8((dp[0] + dp[1]) + (dp[2] + dp[3]));
       // the decayed state's read at k is g kn dot; the write is k_unit u^T = k_raw (kn u)
       const float u = bt * (vv - g * (kn * dot));
       const float uk = kn * u;
-      float po = 0.f;
+      f32x4 pp = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int i4 = 0; i4 < NR / 4; ++i4) {
         const f32x4 q4 = pq[i4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           st[4 * i4 + j] = fmaf(g, st[4 * i4 + j], kr[i4][j] * uk);
-          po = fmaf(q4[j], st[4 * i4 + j], po);
+          pp[j] = fmaf(q4[j], st[4 * i4 + j], pp[j]);
         }
       }
-      po = sum8(po);
+      const float po = sum8((pp[0] + pp[1]) + (pp[2] + pp[3]));
       if (gg == 0) so[tt][cl] = po * qn;
     }
     __syncthreads();
@@ -362,9 +393,15 @@ __global__ __launch_bounds__(512) void delta_scan_kernel(const float* __restrict
   }
   if (live) {
 #pragma unroll
-    for (int i = 0; i < NR; ++i) {
-      const int d = gg * NR + i;
-      if (d < D) S[(long)d * Dv + col] = st[i];
+    for (int i4 = 0; i4 < NR / 4; ++i4) {
+      const int d = gg * NR + 4 * i4;
+      if (vec && d + 3 < D) {
+        *reinterpret_cast<f32x4*>(S + d) = f32x4{st[4 * i4], st[4 * i4 + 1], st[4 * i4 + 2], st[4 * i4 + 3]};
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (d + j < D) S[d + j] = st[4 * i4 + j];
+      }
     }
   }
 }

@@ -212,7 +212,7 @@ def test_delta_rule_through_packed_steps(target, H, G, D, Dv):
     ins = [delta_inputs(n, H, G, D, Dv, 100 * s) for s, n in enumerate(lens)]
     a_log, dt_bias = rnd(H, seed=7, scale=0.7) - 1.0, rnd(H, seed=8)
     want = [delta_want(*ins[s], a_log, dt_bias, D) for s in range(3)]
-    state = torch.full((2, H, D, Dv), 5.0, dtype=torch.float32, device=dev)       # stale: never read at position 0
+    state = torch.full((2, H, Dv, D), 5.0, dtype=torch.float32, device=dev)       # stale: never read at position 0
     slot = [1, 0, 1]
     steps = [[(0, 2), (1, 1)], [(0, 1), (1, 2)], [(0, 35)], [(0, 1), (1, 3)], [(0, 6)],
              [(2, 1)], [(2, 1)], [(2, 19)], [(2, 2)]]
@@ -248,7 +248,7 @@ def test_delta_rule_recalls_a_far_write(target):
     a_log, dt_bias = torch.zeros(H, dtype=F64), torch.zeros(H, dtype=F64)
     want = delta_want(q, k, v, b, a, a_log, dt_bias, D)
     assert (want[-1] - v[0] * D ** -0.5).abs().max() < 1e-3     # the oracle itself recalls it
-    state = torch.zeros(1, H, D, Dv, dtype=torch.float32, device=dev)
+    state = torch.zeros(1, H, Dv, D, dtype=torch.float32, device=dev)
     got = []
     for t in range(T):
         cu, pos = packed_step([(t, 1)], dev)
