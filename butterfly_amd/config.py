@@ -228,10 +228,10 @@ class ModelConfig:
         lp = js.get("loop")
         if lp:
             a, b, times = int(lp["start"]), int(lp["stop"]), int(lp.get("times", 1))
-            if not (0 <= a <= b <= n) or times < 1:
-                raise ValueError("loop: need 0 <= start <= stop <= layers and times >= 1")
-            runs = list(range(a)) + list(range(a, b)) * times + list(range(b, n))
-            start = a if b > a else -1
+            if not (0 <= a <= b <= n) or times < 0:
+                raise ValueError("loop: need 0 <= start <= stop <= layers and times >= 0")
+            runs = list(range(a)) + list(range(a, b)) * times + list(range(b, n))      # (times 0: the span is left out)
+            start = a if (b > a and times > 0) else -1
         mx = lambda key: max([sp.get(key) or 0 for sp in specs] + [0])  # noqa: E731
         moe = [sp["ffn"] for sp in specs if sp["ffn"]]
         return cls(name=name, arch="gevipel", vocab_size=int(js["vocab"]), hidden_size=int(js["width"]),
@@ -316,7 +316,7 @@ def layer_spec(index: int, L: dict) -> dict:
     dim, vdim, taps). `ffn`: None, or kind "dense" (ff) / "glu" (dense clamped GLU with biases: ff,
     limit) / "moe" (ff, limit or None for unclamped experts, experts, top)."""
     m, t = L["mixer"], L["type"]
-    sp = {"index": index, "type": t, "heads": int(m["heads"]), "dim": int(m["dim"]), "vdim": int(m["vdim"]),
+    sp = {"index": index, "type": t, "heads": int(m["heads"]), "dim": int(m["dim"]), "vdim": int(m.get("vdim", m["dim"])),
           "kv_from": None, "kv_heads": 0, "maps": 1}
     if t == "biased_attention":
         qt = m.get("q_temp") or {"coef": 0.0, "every": 1}            # absent: no temperature

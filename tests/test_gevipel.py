@@ -684,6 +684,10 @@ def test_random_init_and_registry():
     assert [len(o) for o in out] == [3, 3]
     with pytest.raises(ValueError):
         ModelConfig.from_gevipel({**cfg_b(), "loop": {"start": 3, "stop": 2, "times": 2}})
+    # a span that runs zero times is left out; one that runs once is the plain order
+    assert ModelConfig.from_gevipel({**cfg_b(), "loop": {"start": 1, "stop": 3, "times": 0}}).layer_runs == [0, 3, 4, 5]
+    once = ModelConfig.from_gevipel({**cfg_b(), "loop": {"start": 1, "stop": 3, "times": 1}})
+    assert once.layer_runs == [0, 1, 2, 3, 4, 5] and build_model(once, device="cpu", dtype=torch.float32).reentry == set()
     bad = cfg_b()
     bad["layers"][1]["mixer"]["vdim"] = 8
     with pytest.raises(ValueError):
